@@ -28,6 +28,48 @@ __global__ void embedding_kernel(const int32_t* __restrict__ tokens, const T* __
   for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = to_f32(src[j]);
 }
 
+// out[t, :] = table[tokens[t], :] * scale + pairs[row(t), :]: a second table indexed by a hash of (the token
+// before, the token), row(t) = (prev * mul_prev + token * mul_cur) mod buckets; a request's first token
+// (position 0) has none before it and takes row `buckets`, the table's last.  The token before the first one a
+// request brings in this step is what its state slot keeps (prev_state[slot], written by the step that brought
+// it); the workgroup of that first token reads it and then leaves the request's last token of this step there,
+// so nobody else touches the slot.
+template <typename T>
+__global__ void embedding_pairs_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ positions,
+                                       const int32_t* __restrict__ req_of_token, const int32_t* __restrict__ cu_seqlens,
+                                       const int32_t* __restrict__ state_slots, int32_t* __restrict__ prev_state,
+                                       const T* __restrict__ table, const T* __restrict__ pairs,
+                                       float* __restrict__ out, int hidden, int vocab, int buckets, int mul_prev,
+                                       int mul_cur, float scale) {
+  const int t = blockIdx.x;
+  const int tok = tokens[t];
+  float* dst = out + (int64_t)t * hidden;
+  if (tok < 0 || tok >= vocab) {  // ids are checked on the host; poison instead of reading outside
+    for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = __builtin_nanf("");
+    return;
+  }
+  const int r = req_of_token[t];
+  const int first = cu_seqlens[r], end = cu_seqlens[r + 1];
+  const bool leads = t == first && t < end;       // padding rows belong to request 0 and lead nothing
+  int prev = 0;
+  if (leads) {
+    const int slot = state_slots[r];
+    prev = prev_state[slot];
+    __syncthreads();                              // every thread has read it
+    if (threadIdx.x == 0) prev_state[slot] = tokens[end - 1];
+  } else if (t > 0) {
+    prev = tokens[t - 1];
+  }
+  int64_t row = buckets;
+  if (positions[t] > 0) {
+    row = ((int64_t)prev * mul_prev + (int64_t)tok * mul_cur) % buckets;
+    if (row < 0) row += buckets;
+  }
+  const T* src = table + (int64_t)tok * hidden;
+  const T* add = pairs + row * hidden;
+  for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = fmaf(to_f32(src[j]), scale, to_f32(add[j]));
+}
+
 // -------------------------------------------------------------------- RMSNorm
 // y = w * x / sqrt(mean(x^2) + eps), statistics in float32.  One workgroup per
 // output row; `rows` (optional) selects the input row of each output row.
@@ -284,6 +326,21 @@ int tl_embedding(const int32_t* tokens, const void* table, float* out, int n_tok
   if (hidden <= 0 || vocab <= 0) return TL_ERR_ARG;
   TL_DISPATCH_T(dtype, hipLaunchKernelGGL(embedding_kernel<T>, dim3(n_tokens), dim3(kThreads), 0, stream,
                                           tokens, (const T*)table, out, hidden, vocab);)
+  return tl_launch_status();
+}
+
+// pairs: [buckets + 1, hidden] of the table's type; prev_state: int32, one per state slot.
+int tl_embedding_pairs(const int32_t* tokens, const int32_t* positions, const int32_t* req_of_token,
+                       const int32_t* cu_seqlens, const int32_t* state_slots, int32_t* prev_state, const void* table,
+                       const void* pairs, float* out, int n_tokens, int hidden, int vocab, int buckets, int mul_prev,
+                       int mul_cur, float scale, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return TL_OK;
+  if (hidden <= 0 || vocab <= 0 || buckets <= 0 || !tokens || !positions || !req_of_token || !cu_seqlens ||
+      !state_slots || !prev_state || !table || !pairs || !out)
+    return TL_ERR_ARG;
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(embedding_pairs_kernel<T>, dim3(n_tokens), dim3(kThreads), 0, stream, tokens,
+                                          positions, req_of_token, cu_seqlens, state_slots, prev_state, (const T*)table,
+                                          (const T*)pairs, out, hidden, vocab, buckets, mul_prev, mul_cur, scale);)
   return tl_launch_status();
 }
 

@@ -18,26 +18,29 @@ constexpr int kMaxQ = 1024;                   // kv_rank + rot
 // [q latent (q_rank) at q_off | kv latent (kv_rank) then the shared key part (rot) at kv_off].
 // cq[t] = w_q * rms_unit(q latent); if the layer keeps a cache of its own (kv_rank > 0):
 // latent[slot] = w_kv * rms_unit(kv latent), rope[slot] = the key part rotated by the angle
-// table's row positions[t] (its first `rdims` dims, pair i with i + rdims/2).  A negative slot stores nothing.
+// table's row positions[t] (its first `rdims` dims; pair i is (i, i + rdims/2), or (2i, 2i + 1) when
+// `interleaved`).  A negative slot stores nothing.  q_rank == 0: there is no query latent.
 template <typename T>
 __global__ void latent_prepare_kernel(const T* __restrict__ d, int64_t d_stride, int q_off, int q_rank, int kv_off,
                                       int kv_rank, int rot, int rdims, const float* __restrict__ w_q,
                                       const float* __restrict__ w_kv, float eps, const int32_t* __restrict__ positions,
                                       const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                       const int32_t* __restrict__ slot_mapping, T* __restrict__ cq,
-                                      T* __restrict__ latent, T* __restrict__ rope) {
+                                      T* __restrict__ latent, T* __restrict__ rope, int interleaved) {
   __shared__ float red[kWaves];
   const int t = blockIdx.x;
   const T* row = d + (int64_t)t * d_stride;
-  float ss = 0.f;
-  for (int j = threadIdx.x; j < q_rank; j += kThreads) {
-    const float v = to_f32(row[q_off + j]);
-    ss += v * v;
+  float ss = 0.f, r = 0.f;
+  if (q_rank > 0) {
+    for (int j = threadIdx.x; j < q_rank; j += kThreads) {
+      const float v = to_f32(row[q_off + j]);
+      ss += v * v;
+    }
+    ss = block_sum<kWaves>(ss, red);
+    r = 1.f / sqrtf(ss / (float)q_rank + eps);
+    for (int j = threadIdx.x; j < q_rank; j += kThreads)
+      cq[(int64_t)t * q_rank + j] = from_f32<T>(to_f32(row[q_off + j]) * r * w_q[j]);
   }
-  ss = block_sum<kWaves>(ss, red);
-  float r = 1.f / sqrtf(ss / (float)q_rank + eps);
-  for (int j = threadIdx.x; j < q_rank; j += kThreads)
-    cq[(int64_t)t * q_rank + j] = from_f32<T>(to_f32(row[q_off + j]) * r * w_q[j]);
   if (kv_rank <= 0) return;
   const int slot = slot_mapping[t];
   ss = 0.f;
@@ -54,21 +57,23 @@ __global__ void latent_prepare_kernel(const T* __restrict__ d, int64_t d_stride,
   const int pos = positions[t];
   for (int i = threadIdx.x; i < half; i += kThreads) {
     const float c = cos_t[(int64_t)pos * half + i], s = sin_t[(int64_t)pos * half + i];
-    const float u = to_f32(row[kv_off + kv_rank + i]), v = to_f32(row[kv_off + kv_rank + half + i]);
-    rope[(int64_t)slot * rot + i] = from_f32<T>(u * c - v * s);
-    rope[(int64_t)slot * rot + half + i] = from_f32<T>(v * c + u * s);
+    const int a = interleaved ? 2 * i : i, b = interleaved ? 2 * i + 1 : half + i;
+    const float u = to_f32(row[kv_off + kv_rank + a]), v = to_f32(row[kv_off + kv_rank + b]);
+    rope[(int64_t)slot * rot + a] = from_f32<T>(u * c - v * s);
+    rope[(int64_t)slot * rot + b] = from_f32<T>(v * c + u * s);
   }
   for (int i = rdims + threadIdx.x; i < rot; i += kThreads)       // dims beyond the rotated ones pass unchanged
     rope[(int64_t)slot * rot + i] = row[kv_off + kv_rank + i];
 }
 
 // out[t, h, out_off + i] (float32) = the `rot` dims at in_off of head h of row t, the first `rdims`
-// of them rotated by the angle table's row positions[t] (pair i with i + rdims/2).
+// of them rotated by the angle table's row positions[t] (pair i is (i, i + rdims/2), or (2i, 2i + 1) when
+// `interleaved`).
 template <typename T>
 __global__ void rotate_into_kernel(const T* __restrict__ q, int64_t q_stride, int head_width, int in_off, int rot,
                                    int rdims, int heads, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
                                    const float* __restrict__ sin_t, float* __restrict__ out, int out_width,
-                                   int out_off) {
+                                   int out_off, int interleaved) {
   const int t = blockIdx.x;
   const int half = rdims / 2, rest = rot - rdims, per_head = half + rest;
   const int pos = positions[t];
@@ -81,24 +86,28 @@ __global__ void rotate_into_kernel(const T* __restrict__ q, int64_t q_stride, in
       continue;
     }
     const float c = cos_t[(int64_t)pos * half + i], s = sin_t[(int64_t)pos * half + i];
-    const float u = to_f32(src[i]), v = to_f32(src[half + i]);
-    dst[i] = u * c - v * s;
-    dst[half + i] = v * c + u * s;
+    const int a = interleaved ? 2 * i : i, b = interleaved ? 2 * i + 1 : half + i;
+    const float u = to_f32(src[a]), v = to_f32(src[b]);
+    dst[a] = u * c - v * s;
+    dst[b] = v * c + u * s;
   }
 }
 
 // One wave64 per (token, head).  Lanes split the keys of a 64-key tile for the scores and the
 // latent's dims for the weighted sum.  The result is multiplied by sigmoid(gate[t, h]) (optional).
+// window > 0: position i sees j with 0 <= i - j < window.  sinks (optional): one number per head whose
+// exponential joins the softmax's denominator (it has no key and no value and is not scaled).
 template <typename T>
 __global__ __launch_bounds__(TL_WAVE) void latent_attention_kernel(
     const float* __restrict__ qa, const T* __restrict__ latent, const T* __restrict__ rope,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ req_of_token,
     const int32_t* __restrict__ positions, const T* __restrict__ gate, int64_t gate_stride, T* __restrict__ out,
-    int heads, int kv_rank, int rot, int block_size, float scale) {
+    int heads, int kv_rank, int rot, int block_size, float scale, int window, const float* __restrict__ sinks) {
   __shared__ float qs[kMaxQ];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = req_of_token[t];
   const int kv_end = positions[t] + 1;
+  const int kv_begin = window > 0 ? max(0, kv_end - window) : 0;
   const int32_t* bt = block_tables + (int64_t)r * max_blocks;
   const int width = kv_rank + rot;
   const float* qrow = qa + ((int64_t)t * heads + h) * width;
@@ -110,7 +119,7 @@ __global__ __launch_bounds__(TL_WAVE) void latent_attention_kernel(
 #pragma unroll
   for (int i = 0; i < kRPL; ++i) o[i] = 0.f;
 
-  for (int base = 0; base < kv_end; base += TL_WAVE) {
+  for (int base = kv_begin; base < kv_end; base += TL_WAVE) {
     const int j = base + lane;
     const bool valid = j < kv_end;
     float s = -INFINITY;
@@ -143,6 +152,10 @@ __global__ __launch_bounds__(TL_WAVE) void latent_attention_kernel(
     m = m_new;
   }
   float f = 1.f / l;
+  if (sinks) {                                        // the sink may lie above every score
+    const float sk = sinks[h], m_fin = fmaxf(m, sk), a = expf(m - m_fin);
+    f = a / (l * a + expf(sk - m_fin));
+  }
   if (gate) f /= 1.f + expf(-to_f32(gate[(int64_t)t * gate_stride + h]));
   T* orow = out + ((int64_t)t * heads + h) * kv_rank;
 #pragma unroll
@@ -175,6 +188,14 @@ typedef short lf_i16x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ bf16x4 lf_read_transposed(const bf16_t* p) {
   return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_i16x4*)p));
 }
+// The factor of an unnormalised output whose running maximum is m (in units of log2 e) and whose sum is l,
+// when exp(sink) joins the denominator: 1 / (l + 2^(sink log2 e - m)), formed so that a sink far above every
+// score overflows nothing.
+__device__ __forceinline__ float with_sink(float m, float l, float sink) {
+  const float sk = sink * 1.44269504088896f, m_fin = fmaxf(m, sk);
+  const float a = __builtin_amdgcn_exp2f(m - m_fin);
+  return a / (l * a + __builtin_amdgcn_exp2f(sk - m_fin));
+}
 __device__ __forceinline__ void lf_wave_sync() {      // a wave's LDS operations are carried out in order
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -187,7 +208,7 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
     const int32_t* __restrict__ tile_tok0, const int32_t* __restrict__ tile_ntok,
     const int32_t* __restrict__ positions, const bf16_t* __restrict__ gate, int64_t gate_stride,
     bf16_t* __restrict__ out, float* __restrict__ part, int n_tokens, int heads, int tpt, int kv_rank, int rot,
-    int block_size, float scale, int n_splits) {
+    int block_size, float scale, int n_splits, int window, const float* __restrict__ sinks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lf_smem[];
   const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE, g = lane / 16, c = lane % 16;
   const int tile = blockIdx.x, head0 = blockIdx.y * 16, split = blockIdx.z;
@@ -238,6 +259,9 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
   const int pos = positions[my_tok];
   const int kv_end = positions[tok0 + ntok - 1] + 1;  // what the tile's last token sees
   const int n_kt = (kv_end + 15) / 16;
+  // the first key tile that the tile's first token still sees through its window
+  const int kt0 = window > 0 ? max(0, positions[tok0] - window + 1) / 16 : 0;
+  const int lowest = window > 0 ? pos - window : -1;  // keys at or before this position are hidden from this row
   const float c_log2 = scale * 1.44269504088896f;
   __syncthreads();
 
@@ -260,7 +284,7 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
 #pragma unroll
   for (int dt = 0; dt < LF_MAXDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int first = split * LF_WAVES + wave, stride = n_splits * LF_WAVES;
+  const int first = kt0 + split * LF_WAVES + wave, stride = n_splits * LF_WAVES;
   if (first < n_kt) fetch(first);
   for (int kt = first; kt < n_kt; kt += stride) {
     // the tile's latents into this wave's LDS area (row c, the chunk this lane holds), and the scores
@@ -282,7 +306,7 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int j = kt * 16 + g * 4 + i;
-      const bool ok = row_valid && j <= pos;
+      const bool ok = row_valid && j <= pos && j > lowest;
       sc[i] = ok ? sc[i] * c_log2 : -INFINITY;
       m_tile = fmaxf(m_tile, sc[i]);
     }
@@ -347,7 +371,7 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
     __syncthreads();
   }
   if (wave != 0 || !row_valid) return;
-  if (n_splits > 1) {                                 // unnormalised, for latent_combine_kernel
+  if (n_splits > 1) {                                 // unnormalised, for latent_combine_kernel (which adds the sink)
     float* prow = part + (((int64_t)split * n_tokens + my_tok) * heads + my_h) * MROW;
 #pragma unroll
     for (int dt = 0; dt < LF_MAXDT; ++dt)
@@ -359,6 +383,7 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
     return;
   }
   float f = l_run > 0.f ? 1.f / l_run : 0.f;
+  if (sinks) f = with_sink(m_run, l_run, sinks[my_h]);
   if (gate) f /= 1.f + expf(-(float)gate[(int64_t)my_tok * gate_stride + my_h]);
   bf16_t* orow = out + ((int64_t)my_tok * heads + my_h) * kv_rank + g * 4;
 #pragma unroll
@@ -385,7 +410,8 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_prefill_bf16_kernel
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ tile_req,
     const int32_t* __restrict__ tile_tok0, const int32_t* __restrict__ tile_ntok,
     const int32_t* __restrict__ positions, const bf16_t* __restrict__ gate, int64_t gate_stride,
-    bf16_t* __restrict__ out, int heads, int tpt, int kv_rank, int rot, int block_size, float scale) {
+    bf16_t* __restrict__ out, int heads, int tpt, int kv_rank, int rot, int block_size, float scale, int window,
+    const float* __restrict__ sinks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lf_smem[];
   const int tid = threadIdx.x, wave = tid / TL_WAVE, lane = tid % TL_WAVE, g = lane / 16, c = lane % 16;
   const int tile = blockIdx.x, head0 = blockIdx.y * 16;
@@ -404,6 +430,12 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_prefill_bf16_kernel
   const int kv_end = positions[tok0 + ntok - 1] + 1;  // what the workgroup's last token sees
   const int wave_end = wave * tpt < ntok ? positions[tok0 + min((wave + 1) * tpt, ntok) - 1] + 1 : 0;
   const int n_kt = (kv_end + LP_KEYS - 1) / LP_KEYS;
+  // through a window the workgroup's first token sees no key before kv_first, this wave's first token none before
+  // wave_first, and this row none at or before `lowest`
+  const int kv_first = window > 0 ? max(0, positions[tok0] - window + 1) : 0;
+  const int wave_first = window > 0 && wave * tpt < ntok ? max(0, positions[tok0 + wave * tpt] - window + 1) : 0;
+  const int lowest = window > 0 ? pos - window : -1;
+  const int kt0 = kv_first / LP_KEYS;
   const float c_log2 = scale * 1.44269504088896f;
 
   // this lane's pieces of its query row, q = hi + lo: the upper terms stay in registers, the lower ones
@@ -471,12 +503,12 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_prefill_bf16_kernel
 #pragma unroll
   for (int dt = 0; dt < LF_MAXDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  lookup(0);
-  fetch(0);
-  if (n_kt > 1) lookup(1);
-  stage(Kl);
+  lookup(kt0);
+  fetch(kt0);
+  if (n_kt > kt0 + 1) lookup(kt0 + 1);
+  stage(Kl + (kt0 & 1) * LP_KEYS * KSTR);
   __syncthreads();
-  for (int kt = 0; kt < n_kt; ++kt) {
+  for (int kt = kt0; kt < n_kt; ++kt) {
     const bf16_t* cur = Kl + (kt & 1) * LP_KEYS * KSTR;
     if (kt + 1 < n_kt) {
       fetch(kt + 1);                                  // on its way while this tile is worked on
@@ -485,7 +517,7 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_prefill_bf16_kernel
 #pragma unroll
     for (int half = 0; half < LP_KEYS / 16; ++half) {
       const int j0 = kt * LP_KEYS + half * 16;
-      if (j0 >= wave_end) continue;                   // no key of these sixteen is seen by this wave's tokens
+      if (j0 >= wave_end || j0 + 16 <= wave_first) continue;      // no key of these sixteen is seen by this wave's tokens
       const bf16_t* rows = cur + half * 16 * KSTR;
       f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -501,7 +533,7 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_prefill_bf16_kernel
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int j = j0 + g * 4 + i;
-        const bool ok = row_valid && j <= pos;
+        const bool ok = row_valid && j <= pos && j > lowest;
         sc[i] = ok ? sc[i] * c_log2 : -INFINITY;
         m_tile = fmaxf(m_tile, sc[i]);
       }
@@ -537,6 +569,7 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_prefill_bf16_kernel
   }
   if (!row_valid) return;
   float f = l_run > 0.f ? 1.f / l_run : 0.f;
+  if (sinks) f = with_sink(m_run, l_run, sinks[my_h]);
   if (gate) f /= 1.f + expf(-(float)gate[(int64_t)my_tok * gate_stride + my_h]);
   bf16_t* orow = out + ((int64_t)my_tok * heads + my_h) * kv_rank + g * 4;
 #pragma unroll
@@ -556,7 +589,8 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_prefill_bf16_kernel
 __global__ __launch_bounds__(TL_WAVE) void latent_combine_kernel(const float* __restrict__ part,
                                                                  const bf16_t* __restrict__ gate, int64_t gate_stride,
                                                                  bf16_t* __restrict__ out, int n_tokens, int heads,
-                                                                 int kv_rank, int n_splits) {
+                                                                 int kv_rank, int n_splits,
+                                                                 const float* __restrict__ sinks) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int MROW = kv_rank + 2;
   const int64_t row = (int64_t)t * heads + h, step = (int64_t)n_tokens * heads;
@@ -567,6 +601,7 @@ __global__ __launch_bounds__(TL_WAVE) void latent_combine_kernel(const float* __
   const float wgt = mine ? __builtin_amdgcn_exp2f(m - M) : 0.f;
   const float L = wave_sum(wgt * l);
   float f = L > 0.f ? 1.f / L : 0.f;
+  if (sinks) f = with_sink(M, L, sinks[h]);
   if (gate) f /= 1.f + expf(-(float)gate[(int64_t)t * gate_stride + h]);
   float acc[kRPL];
 #pragma unroll
@@ -755,6 +790,18 @@ __global__ __launch_bounds__(kThreads) void head_gemm_bf16_kernel(const bf16_t* 
   }
 }
 
+// z[t, c] = a[t, c] * sigmoid(g[t, c]): a gate per element, its pre-activation in the rows of another tensor.
+template <typename T>
+__global__ void gate_rows_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ g, int64_t g_stride,
+                                 T* __restrict__ z, int64_t z_stride, int64_t total, int cols) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / cols;
+  const int c = (int)(i - t * cols);
+  const float gv = to_f32(g[t * g_stride + c]);
+  z[t * z_stride + c] = from_f32<T>(to_f32(a[t * a_stride + c]) / (1.f + expf(-gv)));
+}
+
 }  // namespace
 
 #define TL_DISPATCH_T(dtype, ...)                 \
@@ -768,43 +815,46 @@ extern "C" {
 int tl_latent_prepare(const void* d, int64_t d_stride, int q_off, int q_rank, int kv_off, int kv_rank, int rot,
                       int rdims, const float* w_q, const float* w_kv, float eps, const int32_t* positions, const float* cos_t,
                       const float* sin_t, const int32_t* slot_mapping, void* cq, void* latent, void* rope,
-                      int n_tokens, int dtype, hipStream_t stream) {
+                      int n_tokens, int interleaved, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
-  if (q_rank <= 0 || kv_rank < 0 || rot < 0 || rdims < 0 || rdims % 2 || rdims > rot) return TL_ERR_ARG;
+  if (q_rank < 0 || kv_rank < 0 || q_rank + kv_rank == 0 || rot < 0 || rdims < 0 || rdims % 2 || rdims > rot ||
+      (q_rank > 0 && (!w_q || !cq)) || (interleaved != 0 && interleaved != 1))
+    return TL_ERR_ARG;
   if (kv_rank > 0 && (!slot_mapping || !latent || (rot > 0 && !rope) || (rdims > 0 && (!cos_t || !sin_t || !positions))))
     return TL_ERR_ARG;
   TL_DISPATCH_T(dtype, hipLaunchKernelGGL(latent_prepare_kernel<T>, dim3(n_tokens), dim3(kThreads), 0, stream,
                                           (const T*)d, d_stride, q_off, q_rank, kv_off, kv_rank, rot, rdims, w_q, w_kv, eps,
-                                          positions, cos_t, sin_t, slot_mapping, (T*)cq, (T*)latent, (T*)rope);)
+                                          positions, cos_t, sin_t, slot_mapping, (T*)cq, (T*)latent, (T*)rope,
+                                          interleaved);)
   return tl_launch_status();
 }
 
 int tl_rotate_into(const void* q, int64_t q_stride, int head_width, int in_off, int rot, int rdims, int heads,
                    const int32_t* positions, const float* cos_t, const float* sin_t, float* out, int out_width,
-                   int out_off, int n_tokens, int dtype, hipStream_t stream) {
+                   int out_off, int n_tokens, int interleaved, int dtype, hipStream_t stream) {
   if (n_tokens <= 0 || rot == 0) return TL_OK;
   if (rot < 0 || rdims < 0 || rdims % 2 || rdims > rot || heads <= 0 || in_off + rot > head_width ||
-      out_off + rot > out_width)
+      out_off + rot > out_width || (interleaved != 0 && interleaved != 1))
     return TL_ERR_ARG;
   TL_DISPATCH_T(dtype, hipLaunchKernelGGL(rotate_into_kernel<T>, dim3(n_tokens), dim3(kThreads), 0, stream,
                                           (const T*)q, q_stride, head_width, in_off, rot, rdims, heads, positions, cos_t,
-                                          sin_t, out, out_width, out_off);)
+                                          sin_t, out, out_width, out_off, interleaved);)
   return tl_launch_status();
 }
 
 int tl_latent_attention(const float* qa, const void* latent, const void* rope, const int32_t* block_tables,
                         int max_blocks, const int32_t* req_of_token, const int32_t* positions, const void* gate,
                         int64_t gate_stride, void* out, int n_tokens, int heads, int kv_rank, int rot,
-                        int block_size, float scale, int dtype, hipStream_t stream) {
+                        int block_size, float scale, int window, const float* sinks, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (heads <= 0 || heads > 65535 || kv_rank <= 0 || kv_rank > kMaxRank || rot < 0 || kv_rank + rot > kMaxQ ||
-      block_size <= 0 || max_blocks <= 0)
+      block_size <= 0 || max_blocks <= 0 || window < 0)
     return TL_ERR_ARG;
   dim3 g(n_tokens, heads), b(TL_WAVE);
   TL_DISPATCH_T(dtype, hipLaunchKernelGGL(latent_attention_kernel<T>, g, b, 0, stream, qa, (const T*)latent,
                                           (const T*)rope, block_tables, max_blocks, req_of_token, positions,
                                           (const T*)gate, gate_stride, (T*)out, heads, kv_rank, rot, block_size,
-                                          scale);)
+                                          scale, window, sinks);)
   return tl_launch_status();
 }
 
@@ -815,9 +865,9 @@ int tl_latent_flash(const float* qa, const void* latent, const void* rope, const
                     const int32_t* tile_req, const int32_t* tile_tok0, const int32_t* tile_ntok,
                     const int32_t* positions, const void* gate, int64_t gate_stride, void* out, float* part,
                     int n_tiles, int n_tokens, int heads, int tpt, int kv_rank, int rot, int block_size, float scale,
-                    int n_splits, hipStream_t stream) {
+                    int n_splits, int window, const float* sinks, hipStream_t stream) {
   if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
-  if (heads <= 0 || kv_rank <= 0 || kv_rank % 16 || kv_rank > 16 * LF_MAXDT || rot < 0 || rot % 8 ||
+  if (window < 0 || heads <= 0 || kv_rank <= 0 || kv_rank % 16 || kv_rank > 16 * LF_MAXDT || rot < 0 || rot % 8 ||
       kv_rank + rot > 32 * LF_MAXKS || block_size <= 0 || max_blocks <= 0 || n_splits < 1 || n_splits > TL_WAVE ||
       tpt != 16 / (heads < 16 ? heads : 16) || (n_splits > 1 && !part) || (heads + 15) / 16 > 65535)
     return TL_ERR_ARG;
@@ -833,10 +883,11 @@ int tl_latent_flash(const float* qa, const void* latent, const void* rope, const
   dim3 g(n_tiles, (heads + 15) / 16, n_splits), b(LF_WAVES * TL_WAVE);
   hipLaunchKernelGGL(latent_flash_bf16_kernel, g, b, lds, stream, qa, (const bf16_t*)latent, (const bf16_t*)rope,
                      block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions, (const bf16_t*)gate,
-                     gate_stride, (bf16_t*)out, part, n_tokens, heads, tpt, kv_rank, rot, block_size, scale, n_splits);
+                     gate_stride, (bf16_t*)out, part, n_tokens, heads, tpt, kv_rank, rot, block_size, scale, n_splits,
+                     window, sinks);
   if (n_splits > 1)
     hipLaunchKernelGGL(latent_combine_kernel, dim3(n_tokens, heads), dim3(TL_WAVE), 0, stream, part,
-                       (const bf16_t*)gate, gate_stride, (bf16_t*)out, n_tokens, heads, kv_rank, n_splits);
+                       (const bf16_t*)gate, gate_stride, (bf16_t*)out, n_tokens, heads, kv_rank, n_splits, sinks);
   return tl_launch_status();
 }
 
@@ -844,9 +895,10 @@ int tl_latent_flash(const float* qa, const void* latent, const void* rope, const
 int tl_latent_prefill(const float* qa, const void* latent, const void* rope, const int32_t* block_tables,
                       int max_blocks, const int32_t* tile_req, const int32_t* tile_tok0, const int32_t* tile_ntok,
                       const int32_t* positions, const void* gate, int64_t gate_stride, void* out, int n_tiles,
-                      int heads, int tpt, int kv_rank, int rot, int block_size, float scale, hipStream_t stream) {
+                      int heads, int tpt, int kv_rank, int rot, int block_size, float scale, int window,
+                      const float* sinks, hipStream_t stream) {
   if (n_tiles <= 0) return TL_OK;
-  if (heads <= 0 || kv_rank <= 0 || kv_rank % 16 || kv_rank > 16 * LF_MAXDT || rot < 0 || rot % 8 ||
+  if (window < 0 || heads <= 0 || kv_rank <= 0 || kv_rank % 16 || kv_rank > 16 * LF_MAXDT || rot < 0 || rot % 8 ||
       kv_rank + rot > 32 * LF_MAXKS || block_size <= 0 || max_blocks <= 0 || !tile_req || !tile_tok0 || !tile_ntok ||
       tpt != 16 / (heads < 16 ? heads : 16) || (heads + 15) / 16 > 65535)
     return TL_ERR_ARG;
@@ -863,7 +915,7 @@ int tl_latent_prefill(const float* qa, const void* latent, const void* rope, con
   dim3 g(n_tiles, (heads + 15) / 16), b(LF_WAVES * TL_WAVE);
   hipLaunchKernelGGL(latent_prefill_bf16_kernel, g, b, lds, stream, qa, (const bf16_t*)latent, (const bf16_t*)rope,
                      block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions, (const bf16_t*)gate,
-                     gate_stride, (bf16_t*)out, heads, tpt, kv_rank, rot, block_size, scale);
+                     gate_stride, (bf16_t*)out, heads, tpt, kv_rank, rot, block_size, scale, window, sinks);
   return tl_launch_status();
 }
 
@@ -905,6 +957,18 @@ int tl_head_gemm(const void* in, int64_t in_stride, int in_head_width, const voi
                        (const bf16_t*)w, (bf16_t*)out, out_stride, out_head_width, n_rows, inner, cols);
   else
     return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+// a, g, z: rows of `cols` elements of the engine's type, each with a row stride of its own (z may be a).
+int tl_gate_rows(const void* a, int64_t a_stride, const void* g, int64_t g_stride, void* z, int64_t z_stride,
+                 int n_rows, int cols, int dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (cols <= 0 || a_stride < cols || g_stride < cols || z_stride < cols || !a || !g || !z) return TL_ERR_ARG;
+  const int64_t total = (int64_t)n_rows * cols;
+  dim3 grid((unsigned)ceil_div64(total, kThreads)), b(kThreads);
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(gate_rows_kernel<T>, grid, b, 0, stream, (const T*)a, a_stride, (const T*)g,
+                                          g_stride, (T*)z, z_stride, total, cols);)
   return tl_launch_status();
 }
 

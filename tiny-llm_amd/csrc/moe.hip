@@ -103,19 +103,29 @@ __device__ __forceinline__ void dot_lanes4(const bf16_t* __restrict__ a, const b
 
 __device__ __forceinline__ int expert_of(const int32_t* tokens, const int32_t* table, int t, int j, int top, int vocab,
                                          int experts) {
-  int tok = tokens[t];
+  int tok = tokens ? tokens[t] : t;          // no token ids: the table has a row per token of the step
   tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
   int e = table[(int64_t)tok * top + j];
   return e < 0 ? 0 : (e >= experts ? experts - 1 : e);
 }
 
-// out[t * top + j, n] = sum_k a[t, k] * w[e(t, j)][n, k]
+// What follows an expert's first product: nothing, or the square of max(., 0).
+constexpr int kActNone = 0, kActRelu2 = 1;
+__device__ __forceinline__ float activate(float v, int act) {
+  if (act == kActRelu2) {
+    v = fmaxf(v, 0.f);
+    return v * v;
+  }
+  return v;
+}
+
+// out[t * top + j, n] = act(sum_k a[t, k] * w[e(t, j)][n, k])
 template <typename T>
 __global__ __launch_bounds__(kThreads) void table_moe_up_kernel(const T* __restrict__ a, int64_t a_stride,
                                                                 const T* __restrict__ w,
                                                                 const int32_t* __restrict__ tokens,
                                                                 const int32_t* __restrict__ table, T* __restrict__ out,
-                                                                int top, int experts, int vocab, int N, int K) {
+                                                                int top, int experts, int vocab, int N, int K, int act) {
   const int row = blockIdx.x, t = row / top, j = row - t * top;
   const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
   const int e = expert_of(tokens, table, t, j, top, vocab, experts);
@@ -128,18 +138,19 @@ __global__ __launch_bounds__(kThreads) void table_moe_up_kernel(const T* __restr
     for (int c = 0; c < 4; ++c) wr[c] = we + (int64_t)min(n + c, N - 1) * K;
     float v[4];
     dot_lanes4(arow, wr, K, lane, v);
-    if (lane < 4 && n + lane < N) out[(int64_t)row * N + n + lane] = from_f32<T>(v[lane]);
+    if (lane < 4 && n + lane < N) out[(int64_t)row * N + n + lane] = from_f32<T>(activate(v[lane], act));
   }
 }
 
-// out[t, c] = base[t, c] * base_scale[t] + coef * sum_j sum_k z[t * top + j, k] * w[e(t, j)][c, k]
-// (base and base_scale optional; the experts of a token are added in the table's order)
+// out[t, c] = base[t, c] * base_scale[t] + coef * sum_j row_w[t * top + j] * sum_k z[t * top + j, k] * w[e(t, j)][c, k]
+// (base, base_scale and row_w optional; the experts of a token are added in the table's order)
 template <typename T>
 __global__ __launch_bounds__(kThreads) void table_moe_down_kernel(const T* __restrict__ z, const T* __restrict__ w,
                                                                   const int32_t* __restrict__ tokens,
                                                                   const int32_t* __restrict__ table,
                                                                   const float* __restrict__ base,
                                                                   const float* __restrict__ base_scale,
+                                                                  const float* __restrict__ row_w,
                                                                   float* __restrict__ out, int top, int experts,
                                                                   int vocab, int N, int K, float coef) {
   const int t = blockIdx.x;
@@ -155,8 +166,9 @@ __global__ __launch_bounds__(kThreads) void table_moe_down_kernel(const T* __res
       for (int c = 0; c < 4; ++c) wr[c] = w + ((int64_t)e * N + min(n + c, N - 1)) * K;
       float v[4];
       dot_lanes4(z + ((int64_t)t * top + j) * K, wr, K, lane, v);
+      const float wj = row_w ? row_w[(int64_t)t * top + j] : 1.f;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) acc[c] += v[c];
+      for (int c = 0; c < 4; ++c) acc[c] = fmaf(wj, v[c], acc[c]);
     }
     if (lane < 4 && n + lane < N) {
       const float b = base ? base[(int64_t)t * N + n + lane] * bsc : 0.f;
@@ -249,16 +261,18 @@ __global__ __launch_bounds__(kThreads) void moe_gather_kernel(const bf16_t* __re
   }
 }
 
-// out[t, c] = base[t, c] * base_scale[t] + coef * sum_j y[row_pos[t * top + j], c]
+// out[t, c] = base[t, c] * base_scale[t] + coef * sum_j row_w[t * top + j] * y[row_pos[t * top + j], c]
 __global__ void moe_combine_at_kernel(const float* __restrict__ y, const int32_t* __restrict__ row_pos,
                                       const float* __restrict__ base, const float* __restrict__ base_scale,
-                                      float* __restrict__ out, int64_t total, int N, int top, float coef) {
+                                      const float* __restrict__ row_w, float* __restrict__ out, int64_t total, int N,
+                                      int top, float coef) {
   const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   if (i >= total) return;
   const int64_t t = i / N;
   const int c = (int)(i - t * N);
   float acc = 0.f;
-  for (int j = 0; j < top; ++j) acc += y[(int64_t)row_pos[t * top + j] * N + c];
+  for (int j = 0; j < top; ++j)
+    acc = fmaf(row_w ? row_w[t * top + j] : 1.f, y[(int64_t)row_pos[t * top + j] * N + c], acc);
   const float b = base ? base[i] * (base_scale ? base_scale[t] : 1.f) : 0.f;
   out[i] = fmaf(coef, acc, b);
 }
@@ -331,18 +345,111 @@ __global__ __launch_bounds__(kThreads) void grouped_rows_gemm_bf16_kernel(
   }
 }
 
-// out[t, c] = base[t, c] * base_scale[t] + coef * sum_j y[t * top + j, c]   (the experts in the table's order)
+// out[t, c] = base[t, c] * base_scale[t] + coef * sum_j row_w[t * top + j] * y[t * top + j, c]   (the experts in the
+// table's order)
 __global__ void moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ base,
-                                   const float* __restrict__ base_scale, float* __restrict__ out, int64_t total, int N,
-                                   int top, float coef) {
+                                   const float* __restrict__ base_scale, const float* __restrict__ row_w,
+                                   float* __restrict__ out, int64_t total, int N, int top, float coef) {
   const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   if (i >= total) return;
   const int64_t t = i / N;
   const int c = (int)(i - t * N);
   float acc = 0.f;
-  for (int j = 0; j < top; ++j) acc += y[(t * top + j) * N + c];
+  for (int j = 0; j < top; ++j) acc = fmaf(row_w ? row_w[t * top + j] : 1.f, y[(t * top + j) * N + c], acc);
   const float b = base ? base[i] * (base_scale ? base_scale[t] : 1.f) : 0.f;
   out[i] = fmaf(coef, acc, b);
+}
+
+// ------------------------------------------------------------------------------- a router
+// One wave a token.  z [n_tokens, experts] are the router's logits (float32).  Scores s = softmax(z) over all
+// experts.  The experts lie in `groups` equal runs of neighbours; a run's score is its largest score, and only
+// experts of the `keep` best runs may be chosen (groups <= 1: all may).  The `top` largest scores among those
+// are chosen, largest first (equal scores: the lower index first); ids[t, j] names them, and
+// wts[t, j] = s_j / (sum of the chosen s + 1e-20) * scale.
+constexpr int kMaxRouted = 1024;
+
+struct Best {
+  float v;
+  int i;
+};
+__device__ __forceinline__ Best better(Best a, Best b) { return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a; }
+__device__ __forceinline__ Best wave_best(Best x) {
+#pragma unroll
+  for (int d = TL_WAVE / 2; d >= 1; d >>= 1) {
+    Best o;
+    o.v = __shfl_xor(x.v, d, TL_WAVE);
+    o.i = __shfl_xor(x.i, d, TL_WAVE);
+    x = better(x, o);
+  }
+  return x;
+}
+
+__global__ __launch_bounds__(TL_WAVE) void moe_route_kernel(const float* __restrict__ z, int64_t z_stride,
+                                                            int32_t* __restrict__ ids, float* __restrict__ wts,
+                                                            int experts, int top, int groups, int keep, float scale) {
+  __shared__ float s[kMaxRouted];         // scores; -1 once an expert is chosen or its run is out
+  __shared__ float gs[kMaxRouted];        // the runs' scores
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const float* zr = z + (int64_t)t * z_stride;
+  float m = -INFINITY;
+  for (int e = lane; e < experts; e += TL_WAVE) m = fmaxf(m, zr[e]);
+  m = wave_max(m);
+  float sum = 0.f;
+  for (int e = lane; e < experts; e += TL_WAVE) {
+    const float p = expf(zr[e] - m);
+    s[e] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.f / sum;
+  for (int e = lane; e < experts; e += TL_WAVE) s[e] *= inv;
+  __syncthreads();
+  if (groups > 1 && keep < groups) {
+    const int per = experts / groups;
+    for (int g = lane; g < groups; g += TL_WAVE) {
+      float b = -1.f;
+      for (int e = g * per; e < (g + 1) * per; ++e) b = fmaxf(b, s[e]);
+      gs[g] = b;
+    }
+    __syncthreads();
+    for (int k = 0; k < keep; ++k) {      // the best runs, one a pass; a kept run is marked with -2
+      Best b = {-1.f, 0x7fffffff};
+      for (int g = lane; g < groups; g += TL_WAVE) b = better(b, Best{gs[g], g});
+      b = wave_best(b);
+      __syncthreads();
+      if (lane == 0) gs[b.i] = -2.f;
+      __syncthreads();
+    }
+    for (int e = lane; e < experts; e += TL_WAVE)
+      if (gs[e / per] != -2.f) s[e] = -1.f;
+    __syncthreads();
+  }
+  float total = 0.f;
+  for (int j = 0; j < top; ++j) {         // the best of what is left, one a pass; gs now keeps the chosen scores
+    Best b = {-2.f, 0x7fffffff};
+    for (int e = lane; e < experts; e += TL_WAVE) b = better(b, Best{s[e], e});
+    b = wave_best(b);
+    __syncthreads();
+    if (lane == 0) {
+      s[b.i] = -3.f;
+      gs[j] = b.v;
+      ids[(int64_t)t * top + j] = b.i;
+    }
+    total += b.v;
+    __syncthreads();
+  }
+  const float f = scale / (total + 1e-20f);
+  for (int j = lane; j < top; j += TL_WAVE) wts[(int64_t)t * top + j] = gs[j] * f;
+}
+
+// out[i] = act(in[i]) over rows of `cols` elements (the input's rows may be wider).
+template <typename TI, typename TO>
+__global__ void activate_rows_kernel(const TI* __restrict__ in, int64_t in_stride, TO* __restrict__ out, int64_t total,
+                                     int cols, int act) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / cols;
+  out[i] = from_f32<TO>(activate(to_f32(in[t * in_stride + (i - t * cols)]), act));
 }
 
 }  // namespace
@@ -357,7 +464,7 @@ int tl_moe_plan(const int32_t* tokens, const int32_t* table, int32_t* plan, int 
                 int max_tiles, int rows_a_tile, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   const int64_t rows = (int64_t)n_tokens * top;
-  if (top <= 0 || experts <= 0 || experts > 1024 || vocab <= 0 || rows > 0x7fffffff || !tokens || !table || !plan ||
+  if (top <= 0 || experts <= 0 || experts > 1024 || vocab <= 0 || rows > 0x7fffffff || (!tokens && vocab < n_tokens) || !table || !plan ||
       rows_a_tile <= 0 || max_tiles < (rows + rows_a_tile - 1) / rows_a_tile + experts)
     return TL_ERR_ARG;
   int32_t* counts = plan;
@@ -421,61 +528,64 @@ int tl_moe_gather(const void* a, int64_t a_stride, int a_div, void* dst, int32_t
 }
 
 // As tl_moe_combine with the rows of y looked up in row_pos.
-int tl_moe_combine_at(const float* y, const int32_t* row_pos, const float* base, const float* base_scale, float* out,
-                      int n_tokens, int N, int top, float coef, hipStream_t stream) {
+int tl_moe_combine_at(const float* y, const int32_t* row_pos, const float* base, const float* base_scale,
+                      const float* row_w, float* out, int n_tokens, int N, int top, float coef, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (N <= 0 || top <= 0 || !y || !out || !row_pos) return TL_ERR_ARG;
   const int64_t total = (int64_t)n_tokens * N;
   hipLaunchKernelGGL(moe_combine_at_kernel, dim3((unsigned)ceil_div64(total, kThreads)), dim3(kThreads), 0, stream, y,
-                     row_pos, base, base_scale, out, total, N, top, coef);
+                     row_pos, base, base_scale, row_w, out, total, N, top, coef);
   return tl_launch_status();
 }
 
-int tl_moe_combine(const float* y, const float* base, const float* base_scale, float* out, int n_tokens, int N, int top,
-                   float coef, hipStream_t stream) {
+int tl_moe_combine(const float* y, const float* base, const float* base_scale, const float* row_w, float* out,
+                   int n_tokens, int N, int top, float coef, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (N <= 0 || top <= 0 || !y || !out) return TL_ERR_ARG;
   const int64_t total = (int64_t)n_tokens * N;
   hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)ceil_div64(total, kThreads)), dim3(kThreads), 0, stream, y, base,
-                     base_scale, out, total, N, top, coef);
+                     base_scale, row_w, out, total, N, top, coef);
   return tl_launch_status();
 }
 
-// a: [n_tokens, K] (row stride a_stride); w: [experts, N, K]; table: int32 [vocab, top]; out: [n_tokens * top, N].
+// a: [n_tokens, K] (row stride a_stride); w: [experts, N, K]; table: int32 [vocab, top], looked up by tokens[t], or
+// (tokens null) by t itself; out: [n_tokens * top, N], with the activation `act` (0 none, 1 squared relu) applied.
 int tl_table_moe_up(const void* a, int64_t a_stride, const void* w, const int32_t* tokens, const int32_t* table, void* out,
-                    int n_tokens, int top, int experts, int vocab, int N, int K, int dtype, hipStream_t stream) {
+                    int n_tokens, int top, int experts, int vocab, int N, int K, int act, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
-  if (top <= 0 || experts <= 0 || vocab <= 0 || N <= 0 || K <= 0 || a_stride < K || !a || !w || !tokens || !table || !out ||
+  if (top <= 0 || experts <= 0 || vocab <= 0 || N <= 0 || K <= 0 || a_stride < K || !a || !w || !table || !out ||
+      (act != kActNone && act != kActRelu2) || (!tokens && vocab < n_tokens) ||
       (int64_t)n_tokens * top > 0x7fffffff || (N + kCols - 1) / kCols > 65535)
     return TL_ERR_ARG;
   dim3 g(n_tokens * top, (N + kCols - 1) / kCols), b(kThreads);
   if (dtype == 0)
     hipLaunchKernelGGL(table_moe_up_kernel<float>, g, b, 0, stream, (const float*)a, a_stride, (const float*)w, tokens,
-                       table, (float*)out, top, experts, vocab, N, K);
+                       table, (float*)out, top, experts, vocab, N, K, act);
   else if (dtype == 1)
     hipLaunchKernelGGL(table_moe_up_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)a, a_stride, (const bf16_t*)w, tokens,
-                       table, (bf16_t*)out, top, experts, vocab, N, K);
+                       table, (bf16_t*)out, top, experts, vocab, N, K, act);
   else
     return TL_ERR_ARG;
   return tl_launch_status();
 }
 
 // z: [n_tokens * top, K]; w: [experts, N, K]; base: float32 [n_tokens, N] or null; base_scale: float32 [n_tokens] or
-// null; out: float32 [n_tokens, N] (may be base).
+// null; row_w: float32 [n_tokens * top] or null; out: float32 [n_tokens, N] (may be base).
 int tl_table_moe_down(const void* z, const void* w, const int32_t* tokens, const int32_t* table, const float* base,
-                      const float* base_scale, float* out, int n_tokens, int top, int experts, int vocab, int N, int K,
-                      float coef, int dtype, hipStream_t stream) {
+                      const float* base_scale, const float* row_w, float* out, int n_tokens, int top, int experts,
+                      int vocab, int N, int K, float coef, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
-  if (top <= 0 || experts <= 0 || vocab <= 0 || N <= 0 || K <= 0 || !z || !w || !tokens || !table || !out ||
+  if (top <= 0 || experts <= 0 || vocab <= 0 || N <= 0 || K <= 0 || !z || !w || !table || !out ||
+      (!tokens && vocab < n_tokens) ||
       (N + kCols - 1) / kCols > 65535)
     return TL_ERR_ARG;
   dim3 g(n_tokens, (N + kCols - 1) / kCols), b(kThreads);
   if (dtype == 0)
     hipLaunchKernelGGL(table_moe_down_kernel<float>, g, b, 0, stream, (const float*)z, (const float*)w, tokens, table,
-                       base, base_scale, out, top, experts, vocab, N, K, coef);
+                       base, base_scale, row_w, out, top, experts, vocab, N, K, coef);
   else if (dtype == 1)
     hipLaunchKernelGGL(table_moe_down_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)z, (const bf16_t*)w, tokens, table,
-                       base, base_scale, out, top, experts, vocab, N, K, coef);
+                       base, base_scale, row_w, out, top, experts, vocab, N, K, coef);
   else
     return TL_ERR_ARG;
   return tl_launch_status();
@@ -493,6 +603,35 @@ int tl_row_dot_sigmoid(const void* a, int64_t a_stride, const void* w, float* ou
                        K);
   else
     return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+// z: float32 [n_tokens, experts] (row stride z_stride); ids: int32 [n_tokens, top]; wts: float32 [n_tokens, top].
+int tl_moe_route(const float* z, int64_t z_stride, int32_t* ids, float* wts, int n_tokens, int experts, int top,
+                 int groups, int keep, float scale, hipStream_t stream) {
+  if (n_tokens <= 0) return TL_OK;
+  if (experts <= 0 || experts > kMaxRouted || top <= 0 || top > experts || z_stride < experts || !z || !ids || !wts ||
+      groups < 0 || (groups > 1 && (experts % groups || keep <= 0 || keep > groups || top > keep * (experts / groups))))
+    return TL_ERR_ARG;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(n_tokens), dim3(TL_WAVE), 0, stream, z, z_stride, ids, wts, experts, top,
+                     groups, keep, scale);
+  return tl_launch_status();
+}
+
+// in: [n_rows, >= cols] float32 (dtype_in 0) or bfloat16 (1); out: contiguous [n_rows, cols] in dtype_out.
+int tl_activate_rows(const void* in, int64_t in_stride, void* out, int n_rows, int cols, int act, int dtype_in,
+                     int dtype_out, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (cols <= 0 || in_stride < cols || !in || !out || (act != kActNone && act != kActRelu2)) return TL_ERR_ARG;
+  const int64_t total = (int64_t)n_rows * cols;
+  dim3 g((unsigned)ceil_div64(total, kThreads)), b(kThreads);
+#define TL_ACT(TI, TO) \
+  hipLaunchKernelGGL((activate_rows_kernel<TI, TO>), g, b, 0, stream, (const TI*)in, in_stride, (TO*)out, total, cols, act)
+  if (dtype_in == 0 && dtype_out == 0) TL_ACT(float, float);
+  else if (dtype_in == 0 && dtype_out == 1) TL_ACT(float, bf16_t);
+  else if (dtype_in == 1 && dtype_out == 1) TL_ACT(bf16_t, bf16_t);
+  else return TL_ERR_ARG;
+#undef TL_ACT
   return tl_launch_status();
 }
 

@@ -342,8 +342,11 @@ class ModelRunner:
         readers = decoder.cache_readers()
         for (i, role) in list(decoder.cache_specs()) + list(readers):
             decoder.caches[i][role] = cache.layer_cache((i, role), readers.get((i, role)))
-        for (i, role) in decoder.state_specs():
-            decoder.states[i][role] = cache.states[(i, role)]
+        for owner in decoder.state_specs():
+            if owner == decoder.EMBEDDING_OWNER:
+                decoder.embedding_state = cache.states[owner]
+            else:
+                decoder.states[owner[0]][owner[1]] = cache.states[owner]
         self.workspace = ops.Workspace(self.device, self.max_tokens)
         self._pinned: Optional[torch.Tensor] = None
         self._uploaded: Optional[torch.cuda.Event] = None

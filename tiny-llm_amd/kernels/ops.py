@@ -1137,23 +1137,30 @@ def check_latent_sizes(kv_rank: int, rot: int) -> None:
               f"dims, together at most {LATENT_MAX_QUERY}; got {kv_rank} and {rot}")
 
 
-def latent_prepare(d: torch.Tensor, q_off: int, q_rank: int, w_q: torch.Tensor, eps: float, cq: torch.Tensor,
+def latent_prepare(d: torch.Tensor, q_off: int, q_rank: int, w_q: Optional[torch.Tensor], eps: float,
+                   cq: Optional[torch.Tensor],
                    kv_off: int = 0, kv_rank: int = 0, rot: int = 0, rdims: int = 0,
                    w_kv: Optional[torch.Tensor] = None,
                    positions: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
                    sin: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
-                   latent: Optional[torch.Tensor] = None, rope: Optional[torch.Tensor] = None) -> None:
+                   latent: Optional[torch.Tensor] = None, rope: Optional[torch.Tensor] = None,
+                   pairing: str = "half") -> None:
     """Row t of d holds the down projections.  cq[t] = w_q * unit_rms(d[t, q_off : q_off + q_rank]);
     with kv_rank > 0 also latent[slots[t]] = w_kv * unit_rms(d[t, kv_off : kv_off + kv_rank]) and
     rope[slots[t]] = the next `rot` columns, the first `rdims` of them rotated by the angle tables' row
-    positions[t] (pairs (i, i + rdims/2)).  latent / rope are the paged tensors [blocks, block_size, width]."""
+    positions[t] (pairing "half": pairs (i, i + rdims/2); "interleaved": (2i, 2i + 1)).  latent / rope are the
+    paged tensors [blocks, block_size, width].  q_rank == 0: the layer has no query latent (w_q and cq None)."""
     _dev(d, w_q, cq, w_kv, positions, cos, sin, slots, latent, rope)
     _rows_2d(d, "projections")
     T = d.shape[0]
-    _f32_vec(w_q, q_rank, "the query latent's norm weight")
-    if not (cq.dtype == d.dtype and cq.is_contiguous() and tuple(cq.shape) == (T, q_rank)
-            and 0 <= q_off and q_off + q_rank <= d.shape[1]):
-        _fail("latent_prepare: the query latent must be contiguous [T, q_rank] of the projections' type")
+    _need(pairing in ROPE_PAIRINGS, f"latent_prepare: pairing {pairing!r} is not built")
+    _need(q_rank > 0 or kv_rank > 0, "latent_prepare: nothing to prepare")
+    if q_rank > 0:
+        _need(w_q is not None and cq is not None, "latent_prepare: a query latent needs its norm weight and its output")
+        _f32_vec(w_q, q_rank, "the query latent's norm weight")
+        if not (cq.dtype == d.dtype and cq.is_contiguous() and tuple(cq.shape) == (T, q_rank)
+                and 0 <= q_off and q_off + q_rank <= d.shape[1]):
+            _fail("latent_prepare: the query latent must be contiguous [T, q_rank] of the projections' type")
     if kv_rank > 0:
         _f32_vec(w_kv, kv_rank, "the latent's norm weight")
         _i32(positions, slots)
@@ -1173,16 +1180,18 @@ def latent_prepare(d: torch.Tensor, q_off: int, q_rank: int, w_q: torch.Tensor, 
                                     c_int(kv_rank), c_int(rot), c_int(rdims if kv_rank > 0 else 0), _ptr(w_q), _ptr(w_kv),
                                     c_float(eps), _ptr(positions),
                                     _ptr(cos), _ptr(sin), _ptr(slots), _ptr(cq), _ptr(latent), _ptr(rope), c_int(T),
-                                    c_int(_dt(d)), _stream()), "latent_prepare")
+                                    c_int(ROPE_PAIRINGS.index(pairing)), c_int(_dt(d)), _stream()), "latent_prepare")
 
 
 def rotate_into(q: torch.Tensor, heads: int, head_width: int, in_off: int, rot: int, rdims: int,
                 positions: torch.Tensor,
-                cos: torch.Tensor, sin: torch.Tensor, out: torch.Tensor, out_off: int) -> torch.Tensor:
+                cos: torch.Tensor, sin: torch.Tensor, out: torch.Tensor, out_off: int,
+                pairing: str = "half") -> torch.Tensor:
     """out[t, h, out_off : out_off + rot] (float32) = the dims in_off : in_off + rot of head h of
     row t of q, the first `rdims` of them rotated by the angle tables' row positions[t] (pairs
-    (i, i + rdims/2)), the others as they are."""
+    (i, i + rdims/2), or (2i, 2i + 1) with pairing "interleaved"), the others as they are."""
     _dev(q, positions, cos, sin, out)
+    _need(pairing in ROPE_PAIRINGS, f"rotate_into: pairing {pairing!r} is not built")
     _rows_2d(q, "rotate_into input")
     _i32(positions)
     T = q.shape[0]
@@ -1194,20 +1203,25 @@ def rotate_into(q: torch.Tensor, heads: int, head_width: int, in_off: int, rot: 
         _fail("rotate_into: shapes do not fit")
     _check(_lib().tl_rotate_into(_ptr(q), c_int64(q.stride(0)), c_int(head_width), c_int(in_off), c_int(rot),
                                  c_int(rdims), c_int(heads), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(out), c_int(out.shape[2]),
-                                 c_int(out_off), c_int(T), c_int(_dt(q)), _stream()), "rotate_into")
+                                 c_int(out_off), c_int(T), c_int(ROPE_PAIRINGS.index(pairing)), c_int(_dt(q)), _stream()),
+           "rotate_into")
     return out
 
 
 def latent_attention(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torch.Tensor], block_tables: torch.Tensor,
                      req_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, scale: float,
-                     gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     gate: Optional[torch.Tensor] = None, window: int = 0,
+                     sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """qa float32 [T, heads, kv_rank + rot] = [W_uk^T q_unrotated | q_rotated]; latent / rope the paged
     tensors [blocks, block_size, kv_rank] / [blocks, block_size, rot].  out[t, h] = sigmoid(gate[t, h])
     * sum_j softmax_j((qa[t, h] . [latent_j | rope_j]) * scale) latent_j over the request's positions
-    j <= positions[t].  gate [T, heads] may be a view with a row stride."""
-    _dev(qa, latent, rope, block_tables, req_of_token, positions, out, gate)
+    j <= positions[t].  gate [T, heads] may be a view with a row stride.  window > 0: only the positions
+    j > positions[t] - window.  sinks (float32 [heads]): exp(sinks[h]) joins head h's denominator."""
+    _dev(qa, latent, rope, block_tables, req_of_token, positions, out, gate, sinks)
     _i32(block_tables, req_of_token, positions)
     T, H, W = qa.shape
+    _f32_vec(sinks, H, "latent_attention sinks")
+    _need(window >= 0, "latent_attention: the window is 0 (none) or positive")
     kv_rank = latent.shape[-1]
     rot = W - kv_rank
     check_latent_sizes(kv_rank, rot)
@@ -1226,7 +1240,7 @@ def latent_attention(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torc
                                       c_int(block_tables.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(gate),
                                       c_int64(gate.stride(0) if gate is not None else 0), _ptr(out), c_int(T),
                                       c_int(H), c_int(kv_rank), c_int(rot), c_int(latent.shape[1]), c_float(scale),
-                                      c_int(_dt(latent)), _stream()), "latent_attention")
+                                      c_int(window), _ptr(sinks), c_int(_dt(latent)), _stream()), "latent_attention")
     return out
 
 
@@ -1246,13 +1260,16 @@ def latent_key_splits(groups: int, max_seq_len: int) -> int:
 
 def latent_flash(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torch.Tensor], block_tables: torch.Tensor,
                  tiles, positions: torch.Tensor, out: torch.Tensor, scale: float, gate: Optional[torch.Tensor] = None,
-                 n_splits: int = 1, scratch_buf: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 n_splits: int = 1, scratch_buf: Optional[torch.Tensor] = None, window: int = 0,
+                 sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """`latent_attention` on the matrix cores (bfloat16 caches).  tiles = (tile_req, tile_tok0, tile_ntok)
     with at most 16 // min(heads, 16) tokens of one request each, or None: tile i is token i of request i.
-    n_splits > 1: scratch_buf holds n_splits * T * heads * (kv_rank + 2) floats."""
-    _dev(qa, latent, rope, block_tables, positions, out, gate, scratch_buf)
+    n_splits > 1: scratch_buf holds n_splits * T * heads * (kv_rank + 2) floats.  window, sinks: as there."""
+    _dev(qa, latent, rope, block_tables, positions, out, gate, scratch_buf, sinks)
     _i32(block_tables, positions)
     T, H, W = qa.shape
+    _f32_vec(sinks, H, "latent_flash sinks")
+    _need(window >= 0, "latent_flash: the window is 0 (none) or positive")
     kv_rank = latent.shape[-1]
     rot = W - kv_rank
     if not latent_flash_supported(latent.dtype, kv_rank, rot):
@@ -1288,7 +1305,7 @@ def latent_flash(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torch.Te
                                   _ptr(gate), c_int64(gate.stride(0) if gate is not None else 0), _ptr(out, 8),
                                   _ptr(scratch_buf, 16), c_int(n_tiles), c_int(T), c_int(H), c_int(16 // min(H, 16)),
                                   c_int(kv_rank), c_int(rot), c_int(latent.shape[1]), c_float(scale),
-                                  c_int(n_splits), _stream()), "latent_flash")
+                                  c_int(n_splits), c_int(window), _ptr(sinks), _stream()), "latent_flash")
     return out
 
 
@@ -1297,13 +1314,16 @@ LATENT_PREFILL_ROWS = 64        # from this many query rows on a step's latent a
 
 def latent_prefill(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torch.Tensor], block_tables: torch.Tensor,
                    tiles, positions: torch.Tensor, out: torch.Tensor, scale: float,
-                   gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   gate: Optional[torch.Tensor] = None, window: int = 0,
+                   sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """`latent_flash` for steps with many query rows: tiles = (tile_req, tile_tok0, tile_ntok) with at most
     4 * (16 // min(heads, 16)) tokens of one request each; the four waves of a workgroup share every staged
     key tile.  Same operands and result otherwise (no split keys)."""
-    _dev(qa, latent, rope, block_tables, positions, out, gate)
+    _dev(qa, latent, rope, block_tables, positions, out, gate, sinks)
     _i32(block_tables, positions)
     T, H, W = qa.shape
+    _f32_vec(sinks, H, "latent_prefill sinks")
+    _need(window >= 0, "latent_prefill: the window is 0 (none) or positive")
     kv_rank = latent.shape[-1]
     rot = W - kv_rank
     if not latent_flash_supported(latent.dtype, kv_rank, rot):
@@ -1329,7 +1349,8 @@ def latent_prefill(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torch.
                                     c_int(block_tables.shape[1]), _ptr(treq), _ptr(ttok), _ptr(tn), _ptr(positions),
                                     _ptr(gate), c_int64(gate.stride(0) if gate is not None else 0), _ptr(out, 8),
                                     c_int(n_tiles), c_int(H), c_int(16 // min(H, 16)), c_int(kv_rank), c_int(rot),
-                                    c_int(latent.shape[1]), c_float(scale), _stream()), "latent_prefill")
+                                    c_int(latent.shape[1]), c_float(scale), c_int(window), _ptr(sinks), _stream()),
+           "latent_prefill")
     return out
 
 
@@ -1755,32 +1776,48 @@ def tanh_rows(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 
 
 # ------------------------------------------------------------ experts looked up in a table
-def table_moe_up(a: torch.Tensor, w: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t * top + j] = w[table[tokens[t], j]] @ a[t]; a [T, K], w [E, N, K] of one type, table int32 [vocab, top],
-    out contiguous [T * top, N]."""
+MOE_ACTIVATIONS = {None: 0, "relu2": 1}      # what may follow an expert's first product (csrc/moe.hip)
+
+
+def table_moe_up(a: torch.Tensor, w: torch.Tensor, tokens: Optional[torch.Tensor], table: torch.Tensor, out: torch.Tensor,
+                 act: Optional[str] = None) -> torch.Tensor:
+    """out[t * top + j] = act(w[table[tokens[t], j]] @ a[t]); a [T, K], w [E, N, K] of one type, table int32 [vocab, top],
+    out contiguous [T * top, N].  tokens None: the table has a row per row of a (the experts a router chose).
+    act None or "relu2" (the square of max(., 0))."""
     _dev(a, w, tokens, table, out)
+    _need(act in MOE_ACTIVATIONS, f"table_moe_up: activation {act!r} is not built")
     _rows_2d(a, "table_moe_up input")
     T, K = a.shape
     E, N, _ = w.shape
     V, top = table.shape
     _need(w.is_contiguous() and w.shape[2] == K and w.dtype == a.dtype == out.dtype, "table_moe_up: w is contiguous [E, N, K]")
     _need(out.is_contiguous() and tuple(out.shape) == (T * top, N), "table_moe_up: the output is contiguous [T * top, N]")
-    _i32(tokens, table)
-    _need(tokens.numel() == T, "table_moe_up: one token id per row")
+    _i32(table)
+    if tokens is not None:
+        _i32(tokens)
+        _need(tokens.numel() == T, "table_moe_up: one token id per row")
+    else:
+        _need(V >= T and table.is_contiguous(), "table_moe_up: without token ids the table has a row per row of the input")
     _check(_lib().tl_table_moe_up(_ptr(a), c_int64(a.stride(0)), _ptr(w), _ptr(tokens), _ptr(table), _ptr(out), c_int(T),
-                                  c_int(top), c_int(E), c_int(V), c_int(N), c_int(K), c_int(_dt(a)), _stream()),
-           "table_moe_up")
+                                  c_int(top), c_int(E), c_int(V), c_int(N), c_int(K), c_int(MOE_ACTIVATIONS[act]),
+                                  c_int(_dt(a)), _stream()), "table_moe_up")
     return out
 
 
-def table_moe_down(z: torch.Tensor, w: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor,
-                   coef: float, base: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = base[t] * base_scale[t] + coef * sum_j w[table[tokens[t], j]] @ z[t * top + j]; z [T * top, K],
-    w [E, N, K], out float32 [T, N] (may be base); base float32 [T, N], base_scale float32 [T], both optional."""
-    _dev(z, w, tokens, table, out, base, base_scale)
+def table_moe_down(z: torch.Tensor, w: torch.Tensor, tokens: Optional[torch.Tensor], table: torch.Tensor,
+                   out: torch.Tensor, coef: float, base: Optional[torch.Tensor] = None,
+                   base_scale: Optional[torch.Tensor] = None, row_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = base[t] * base_scale[t] + coef * sum_j row_weights[t, j] * w[table[tokens[t], j]] @ z[t * top + j];
+    z [T * top, K], w [E, N, K], out float32 [T, N] (may be base); base float32 [T, N], base_scale float32 [T],
+    row_weights float32 [T, top], all three optional.  tokens None: the table has a row per token of the step."""
+    _dev(z, w, tokens, table, out, base, base_scale, row_weights)
     E, N, K = w.shape
     V, top = table.shape
-    T = tokens.numel()
+    T = tokens.numel() if tokens is not None else out.shape[0]
+    if tokens is None:
+        _need(V >= T and table.is_contiguous(), "table_moe_down: without token ids the table has a row per token")
+    if row_weights is not None:
+        _f32_vec(row_weights, T * top, "table_moe_down row_weights")
     _need(w.is_contiguous() and z.is_contiguous() and tuple(z.shape) == (T * top, K) and z.dtype == w.dtype,
           "table_moe_down: z is contiguous [T * top, K], w contiguous [E, N, K]")
     _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, N),
@@ -1790,8 +1827,11 @@ def table_moe_down(z: torch.Tensor, w: torch.Tensor, tokens: torch.Tensor, table
               "table_moe_down: base is contiguous float32 [T, N]")
     if base_scale is not None:
         _f32_vec(base_scale, T, "table_moe_down base_scale")
-    _i32(tokens, table)
-    _check(_lib().tl_table_moe_down(_ptr(z), _ptr(w), _ptr(tokens), _ptr(table), _ptr(base), _ptr(base_scale), _ptr(out),
+    _i32(table)
+    if tokens is not None:
+        _i32(tokens)
+    _check(_lib().tl_table_moe_down(_ptr(z), _ptr(w), _ptr(tokens), _ptr(table), _ptr(base), _ptr(base_scale),
+                                    _ptr(row_weights), _ptr(out),
                                     c_int(T), c_int(top), c_int(E), c_int(V), c_int(N), c_int(K), c_float(coef),
                                     c_int(_dt(z)), _stream()), "table_moe_down")
     return out
@@ -1812,17 +1852,22 @@ def moe_plan_ints(rows: int, experts: int, tile_rows: int = MOE_TILE_ROWS) -> in
     return 3 * experts + 2 + 3 * moe_max_tiles(rows, experts, tile_rows) + rows
 
 
-def moe_plan(tokens: torch.Tensor, table: torch.Tensor, plan: torch.Tensor, experts: int,
-             tile_rows: int = MOE_TILE_ROWS) -> torch.Tensor:
+def moe_plan(tokens: Optional[torch.Tensor], table: torch.Tensor, plan: torch.Tensor, experts: int,
+             tile_rows: int = MOE_TILE_ROWS, num_tokens: Optional[int] = None) -> torch.Tensor:
     """Sorts the step's rows (token t, its j-th expert: row t * top + j) by expert on the device and lists
     tiles of at most `tile_rows` rows of one expert each; `plan` is int32 scratch of `moe_plan_ints` elements:
     counts[E], cursors[E], offsets[E + 1], the number of tiles, then per tile (capacity `moe_max_tiles`) its
     expert (-1 behind the last tile), its first place in the sorted rows and its number of rows, then the rows
-    sorted by expert."""
+    sorted by expert.  tokens None: the table has a row per token of the step, `num_tokens` of them."""
     _dev(tokens, table, plan)
-    _i32(tokens, table, plan)
+    _i32(table, plan)
     V, top = table.shape
-    T = tokens.numel()
+    if tokens is not None:
+        _i32(tokens)
+        T = tokens.numel()
+    else:
+        T = int(num_tokens)
+        _need(0 < T <= V and table.is_contiguous(), "moe_plan: without token ids the table has a row per token")
     _need(plan.numel() >= moe_plan_ints(T * top, experts, tile_rows), "moe_plan: the plan is too short")
     _need(0 < experts <= 1024, "moe_plan: 1 to 1024 experts")
     plan[:2 * experts].zero_()          # counts and cursors (a fill kernel: fine inside a captured step)
@@ -1882,10 +1927,14 @@ def linear_grouped(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, o
 
 
 def moe_combine_at(y: torch.Tensor, row_pos: torch.Tensor, out: torch.Tensor, top: int, coef: float,
-                   base: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = base[t] * base_scale[t] + coef * sum_j y[row_pos[t * top + j]]; y float32 [*, N], out float32 [T, N]."""
-    _dev(y, row_pos, out, base, base_scale)
+                   base: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None,
+                   row_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = base[t] * base_scale[t] + coef * sum_j row_weights[t, j] * y[row_pos[t * top + j]]; y float32 [*, N],
+    out float32 [T, N]; row_weights float32 [T, top], optional."""
+    _dev(y, row_pos, out, base, base_scale, row_weights)
     T, N = out.shape
+    if row_weights is not None:
+        _f32_vec(row_weights, T * top, "moe_combine_at row_weights")
     _need(out.dtype == torch.float32 and out.is_contiguous(), "moe_combine_at: out is contiguous float32 [T, N]")
     _need(y.dtype == torch.float32 and y.is_contiguous() and y.dim() == 2 and y.shape[1] == N,
           "moe_combine_at: y is contiguous float32 [*, N]")
@@ -1896,7 +1945,8 @@ def moe_combine_at(y: torch.Tensor, row_pos: torch.Tensor, out: torch.Tensor, to
               "moe_combine_at: base is contiguous float32 [T, N]")
     if base_scale is not None:
         _f32_vec(base_scale, T, "moe_combine_at base_scale")
-    _check(_lib().tl_moe_combine_at(_ptr(y), _ptr(row_pos), _ptr(base), _ptr(base_scale), _ptr(out), c_int(T), c_int(N),
+    _check(_lib().tl_moe_combine_at(_ptr(y), _ptr(row_pos), _ptr(base), _ptr(base_scale), _ptr(row_weights), _ptr(out),
+                                    c_int(T), c_int(N),
                                     c_int(top), c_float(coef), _stream()), "moe_combine_at")
     return out
 
@@ -1922,10 +1972,13 @@ def grouped_rows_gemm(a: torch.Tensor, a_div: int, w: torch.Tensor, plan: torch.
 
 
 def moe_combine(y: torch.Tensor, out: torch.Tensor, top: int, coef: float, base: Optional[torch.Tensor] = None,
-                base_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = base[t] * base_scale[t] + coef * sum_j y[t * top + j]; all float32, out may be base."""
-    _dev(y, out, base, base_scale)
+                base_scale: Optional[torch.Tensor] = None, row_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = base[t] * base_scale[t] + coef * sum_j row_weights[t, j] * y[t * top + j]; all float32, out may be
+    base; row_weights [T, top], optional."""
+    _dev(y, out, base, base_scale, row_weights)
     T, N = out.shape
+    if row_weights is not None:
+        _f32_vec(row_weights, T * top, "moe_combine row_weights")
     _need(out.dtype == torch.float32 and out.is_contiguous(), "moe_combine: out is contiguous float32 [T, N]")
     _f32_vec(y, T * top * N, "moe_combine input")
     if base is not None:
@@ -1933,7 +1986,8 @@ def moe_combine(y: torch.Tensor, out: torch.Tensor, top: int, coef: float, base:
               "moe_combine: base is contiguous float32 [T, N]")
     if base_scale is not None:
         _f32_vec(base_scale, T, "moe_combine base_scale")
-    _check(_lib().tl_moe_combine(_ptr(y), _ptr(base), _ptr(base_scale), _ptr(out), c_int(T), c_int(N), c_int(top),
+    _check(_lib().tl_moe_combine(_ptr(y), _ptr(base), _ptr(base_scale), _ptr(row_weights), _ptr(out), c_int(T), c_int(N),
+                                 c_int(top),
                                  c_float(coef), _stream()), "moe_combine")
     return out
 
@@ -1947,4 +2001,80 @@ def row_dot_sigmoid(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torc
     _f32_vec(out, T, "row_dot_sigmoid output")
     _check(_lib().tl_row_dot_sigmoid(_ptr(a), c_int64(a.stride(0)), _ptr(w), _ptr(out), c_int(T), c_int(K),
                                      c_int(_dt(a)), _stream()), "row_dot_sigmoid")
+    return out
+
+
+MOE_MAX_ROUTED = 1024       # experts the router kernel takes (csrc/moe.hip)
+
+
+def moe_route(z: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, groups: int = 1, keep: int = 1,
+              scale: float = 1.0) -> None:
+    """A router over the logits z (float32 [T, E], rows may be wider apart): scores s = softmax(z) over all experts;
+    the experts lie in `groups` equal runs of neighbours, a run's score is its largest, and only experts of the
+    `keep` best runs may be chosen (groups <= 1: all may); ids[t] (int32 [T, top]) names the `top` largest scores
+    among those, largest first (equal scores: the lower index first), and weights[t] (float32 [T, top]) =
+    their scores / (their sum + 1e-20) * scale."""
+    _dev(z, ids, weights)
+    _rows_2d(z, "moe_route logits")
+    T, E = z.shape
+    top = ids.shape[1] if ids.dim() == 2 else 0
+    _need(z.dtype == torch.float32, "moe_route: logits are float32")
+    _need(ids.dtype == torch.int32 and ids.is_contiguous() and tuple(ids.shape) == (T, top) and top > 0,
+          "moe_route: ids are contiguous int32 [T, top]")
+    _f32_vec(weights, T * top, "moe_route weights")
+    _need(0 < top <= E <= MOE_MAX_ROUTED, f"moe_route: 1 to {MOE_MAX_ROUTED} experts, top within them")
+    if groups > 1:
+        _need(E % groups == 0 and 0 < keep <= groups and top <= keep * (E // groups),
+              "moe_route: equal groups, 1 to `groups` of them kept, holding at least `top` experts")
+    _check(_lib().tl_moe_route(_ptr(z), c_int64(z.stride(0)), _ptr(ids), _ptr(weights), c_int(T), c_int(E), c_int(top),
+                               c_int(groups), c_int(keep), c_float(scale), _stream()), "moe_route")
+
+
+def activate_rows(x: torch.Tensor, out: torch.Tensor, act: Optional[str]) -> torch.Tensor:
+    """out = act(x) element by element (act as in `table_moe_up`); x [T, N] float32 or of out's type, its rows may be
+    wider apart; out contiguous [T, N]."""
+    _dev(x, out)
+    _rows_2d(x, "activate_rows input")
+    _need(act in MOE_ACTIVATIONS, f"activate_rows: activation {act!r} is not built")
+    _need(out.is_contiguous() and out.shape == x.shape and (x.dtype == out.dtype or x.dtype == torch.float32),
+          "activate_rows: out is contiguous, of the input's shape, and of its type unless the input is float32")
+    _check(_lib().tl_activate_rows(_ptr(x), c_int64(x.stride(0)), _ptr(out), c_int(x.shape[0]), c_int(x.shape[1]),
+                                   c_int(MOE_ACTIVATIONS[act]), c_int(_dt(x)), c_int(_dt(out)), _stream()), "activate_rows")
+    return out
+
+
+def gate_rows(a: torch.Tensor, g: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = a * sigmoid(g) element by element; a, g, out [T, N] of one type, each may be a view into wider rows
+    (out may be a)."""
+    _dev(a, g, out)
+    for t, name in ((a, "gate_rows input"), (g, "gate_rows gate"), (out, "gate_rows output")):
+        _rows_2d(t, name)
+    _need(a.shape == g.shape == out.shape and a.dtype == g.dtype == out.dtype, "gate_rows: one shape and one type")
+    _check(_lib().tl_gate_rows(_ptr(a), c_int64(a.stride(0)), _ptr(g), c_int64(g.stride(0)), _ptr(out),
+                               c_int64(out.stride(0)), c_int(a.shape[0]), c_int(a.shape[1]), c_int(_dt(a)), _stream()),
+           "gate_rows")
+    return out
+
+
+def embedding_pairs(tokens: torch.Tensor, positions: torch.Tensor, req_of_token: torch.Tensor, cu_seqlens: torch.Tensor,
+                    state_slots: torch.Tensor, prev_state: torch.Tensor, table: torch.Tensor, pairs: torch.Tensor,
+                    out: torch.Tensor, mul_prev: int, mul_cur: int, scale: float) -> torch.Tensor:
+    """out[t] = table[tokens[t]] * scale + pairs[(prev * mul_prev + tokens[t] * mul_cur) mod buckets] as float32,
+    `prev` the token before it in its request; a request's first token (position 0) takes the last row of pairs
+    ([buckets + 1, H]).  prev_state (int32, one element per state slot) keeps every request's last token between
+    steps: read for the first token a request brings, then overwritten with the last one it brings."""
+    _dev(tokens, positions, req_of_token, cu_seqlens, state_slots, prev_state, table, pairs, out)
+    _i32(tokens, positions, req_of_token, cu_seqlens, state_slots, prev_state)
+    T = tokens.numel()
+    V, H = table.shape
+    _need(table.is_contiguous() and pairs.is_contiguous() and pairs.dtype == table.dtype and pairs.dim() == 2
+          and pairs.shape[1] == H and pairs.shape[0] >= 2, "embedding_pairs: tables are contiguous [rows, H] of one type")
+    _need(positions.numel() == T and req_of_token.numel() == T, "embedding_pairs: one position and request per token")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H),
+          f"embedding_pairs: the output is float32 [{T}, {H}]")
+    _need(abs(int(mul_prev)) < (1 << 31) and abs(int(mul_cur)) < (1 << 31), "embedding_pairs: multipliers fit 32 bits")
+    _check(_lib().tl_embedding_pairs(_ptr(tokens), _ptr(positions), _ptr(req_of_token), _ptr(cu_seqlens),
+                                     _ptr(state_slots), _ptr(prev_state), _ptr(table), _ptr(pairs), _ptr(out), c_int(T),
+                                     c_int(H), c_int(V), c_int(pairs.shape[0] - 1), c_int(int(mul_prev)),
+                                     c_int(int(mul_cur)), c_float(scale), c_int(_dt(table)), _stream()), "embedding_pairs")
     return out

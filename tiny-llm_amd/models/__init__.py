@@ -1,2 +1,2 @@
-from . import llama, lufazen, fofapel  # noqa: F401  (register LlamaForCausalLM, Lufazen, Fofapel)
+from . import llama, lufazen, fofapel, gesutar  # noqa: F401  (register LlamaForCausalLM, Lufazen, Fofapel, Gesutar)
 from .decoder import Decoder

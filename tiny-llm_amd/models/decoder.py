@@ -68,6 +68,7 @@ class Decoder:
         # cache and state views by role, per plan entry; attached by the runner once the pools exist
         self.caches: List[Dict[str, LayerCache]] = [{} for _ in spec.plan]
         self.states: List[Dict[str, torch.Tensor]] = [{} for _ in spec.plan]
+        self.embedding_state: Optional[torch.Tensor] = None     # if the embedding keeps per-request state
         self._graph_safe: Optional[bool] = None
         self._graph_runs: Optional[List[tuple]] = None
 
@@ -118,8 +119,12 @@ class Decoder:
                     out[(i, role)] = (e.cache_of, role)
         return out
 
+    EMBEDDING_OWNER: Owner = (-1, "embedding")      # who owns the embedding's per-request state
+
     def state_specs(self) -> Dict[Owner, StateSpec]:
         out: Dict[Owner, StateSpec] = {}
+        if self.embedding.state_spec() is not None:
+            out[self.EMBEDDING_OWNER] = self.embedding.state_spec()
         for i, e in enumerate(self.spec.plan):
             for role, part in self.layers[e.layer].by_role.items():
                 ss = part.state_spec()
@@ -174,7 +179,10 @@ class Decoder:
         # a head that says so may receive the final norm unevaluated and fuse it into its product
         lazy_head = hasattr(self.final_norm, "lazy") and getattr(self.lm_head, "accepts_lazy_norm", False)
         if first == 0:
-            x = self.embedding.forward(ctx.tokens, ctx)
+            if self.embedding_state is not None:
+                x = self.embedding.forward(ctx.tokens, ctx, state=self.embedding_state)
+            else:
+                x = self.embedding.forward(ctx.tokens, ctx)
         # A block may prepare the norm that reads its result (the next block's first norm, or the
         # final norm) in its last product; `prepared` carries that from one block to the next.
         prepared = None

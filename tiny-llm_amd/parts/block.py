@@ -17,12 +17,16 @@ class StreamCopyWanted:
 
 
 class PreNormBlock(Block):
+    """x + mixer(norm(x)), then x + ffn(norm(x)); a layer may have no feed-forward (and then no second norm)."""
     roles = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "ffn": "feed_forward"}
+    optional = ("ffn_norm", "ffn")
 
     def __init__(self, parts):
         super().__init__(parts)
         self.mixer_norm, self.mixer = parts["mixer_norm"], parts["mixer"]
-        self.ffn_norm, self.ffn = parts["ffn_norm"], parts["ffn"]
+        self.ffn_norm, self.ffn = parts.get("ffn_norm"), parts.get("ffn")
+        if (self.ffn is None) != (self.ffn_norm is None):
+            raise ValueError("pre_norm: a feed-forward comes with its norm, and the norm with a feed-forward")
 
     def forward(self, x, ctx, caches, states):
         return self.forward_chained(x, ctx, caches, states)[0]
@@ -37,8 +41,11 @@ class PreNormBlock(Block):
         product that wrote x (or None); `next_norm` is the norm that will read this block's result
         (or None).  Returns (x, that norm prepared or None)."""
         h = self._normed(self.mixer_norm, self.mixer, x, prepared)
+        mixer_args = (h, ctx, caches.get("mixer"), states.get("mixer"), x)
+        if self.ffn is None:
+            return self._run(self.mixer, mixer_args, next_norm)
         ffn_norm = self.ffn_norm if getattr(self.ffn, "accepts_lazy_norm", False) else None
-        x, prep = self._run(self.mixer, (h, ctx, caches.get("mixer"), states.get("mixer"), x), ffn_norm)
+        x, prep = self._run(self.mixer, mixer_args, ffn_norm)
         h = self._normed(self.ffn_norm, self.ffn, x, prep)
         return self._run(self.ffn, (h, ctx, x), next_norm)
 

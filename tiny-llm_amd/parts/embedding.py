@@ -9,7 +9,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..kernels import ops
-from .base import Embedding, Head, WeightSpec, register_embedding, register_head
+from .base import Embedding, Head, StateSpec, WeightSpec, register_embedding, register_head
 from .norm import LazyNorm
 
 
@@ -31,6 +31,46 @@ class TokenEmbedding(Embedding):
     def forward(self, tokens: torch.Tensor, ctx=None) -> torch.Tensor:
         out = ops.scratch("residual", (tokens.numel(), self.hidden_size), torch.float32, tokens.device)
         return ops.embedding(tokens, self.weight, out)
+
+
+class PairEmbedding(Embedding):
+    """x = table[token] * scale + pairs[(previous token * mul_prev + token * mul_cur) mod buckets]: a second
+    table of `buckets` + 1 rows looked up by a hash of the token and the one before it in its request; a
+    request's first token has none before it and takes the last row.  The previous token is per-request
+    state: one int32 per state slot, read for the first token a request brings in a step and overwritten
+    with the last one it brings (the decoder hands the state tensor to `forward`)."""
+    graph_safe = True
+
+    def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int, buckets: int, mul_prev: int,
+                 mul_cur: int, scale: float = 1.0, weight_name: str = "weight", pairs_name: str = "pairs"):
+        """pairs_name: the pair table's tensor name (whole, not below the prefix)."""
+        super().__init__(prefix, dtype, device)
+        self.vocab_size, self.hidden_size, self.buckets = int(vocab_size), int(hidden_size), int(buckets)
+        self.mul_prev, self.mul_cur, self.scale = int(mul_prev), int(mul_cur), float(scale)
+        if self.buckets <= 0:
+            raise ValueError(f"{prefix}: the pair table needs at least one bucket")
+        self.tensor_name = f"{prefix}.{weight_name}" if weight_name else prefix
+        self.pairs_name = pairs_name
+        self.weight: Optional[torch.Tensor] = None
+        self.pairs: Optional[torch.Tensor] = None
+
+    def weights(self) -> List[WeightSpec]:
+        return [WeightSpec(self.tensor_name, (self.vocab_size, self.hidden_size)),
+                WeightSpec(self.pairs_name, (self.buckets + 1, self.hidden_size))]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.tensor_name].contiguous()
+        self.pairs = tensors[self.pairs_name].contiguous()
+
+    def state_spec(self) -> StateSpec:
+        return StateSpec((1,), torch.int32)
+
+    def forward(self, tokens: torch.Tensor, ctx=None, state: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if ctx is None or state is None:
+            raise ValueError(f"{self.prefix}: the pair table needs the step's context and the requests' state")
+        out = ops.scratch("residual", (tokens.numel(), self.hidden_size), torch.float32, tokens.device)
+        return ops.embedding_pairs(tokens, ctx.positions, ctx.req_of_token, ctx.cu_seqlens_q, ctx.state_slots, state,
+                                   self.weight, self.pairs, out, self.mul_prev, self.mul_cur, self.scale)
 
 
 class LMHead(Head):
@@ -69,4 +109,5 @@ class LMHead(Head):
 
 
 register_embedding("token_embedding", TokenEmbedding)
+register_embedding("pair_embedding", PairEmbedding)
 register_head("lm_head", LMHead)

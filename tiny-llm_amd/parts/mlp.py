@@ -139,6 +139,49 @@ class GeluGLU(FeedForward):
         return ops.linear(z, self.w_down, residual, residual)
 
 
+class ActMLP(FeedForward):
+    """down(act(up(h))): a feed-forward without a gate.  act "relu2" is the square of max(., 0).  The up
+    product leaves float32 and the activation rounds once to the engine's element type for the down
+    product.  `names`: the tensors' names below the prefix, (up, down).  With `residual=None` the result
+    is returned by itself in float32."""
+    graph_safe = True
+
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, intermediate_size: int, activation: str = "relu2",
+                 names=("up", "down")):
+        super().__init__(prefix, dtype, device)
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        if activation not in ops.MOE_ACTIVATIONS or activation is None:
+            raise ValueError(f"{prefix}: activation {activation!r} is not built; known: relu2")
+        self.activation = activation
+        ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
+        ops.check_linear_sizes(dtype, self.intermediate_size, f"{prefix}: intermediate_size")
+        self.names = tuple(f"{prefix}.{n}" for n in names)
+        self.w_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def weights(self) -> List[WeightSpec]:
+        H, I = self.hidden_size, self.intermediate_size
+        up, down = self.names
+        return [WeightSpec(up, (I, H)), WeightSpec(down, (H, I))]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        up, down = self.names
+        self.w_up = tensors[up].contiguous()
+        self.w_down = tensors[down].contiguous()
+
+    def forward(self, h, ctx, residual):
+        T, dev = h.shape[0], h.device
+        u = ops.scratch("ffn_up", (T, self.intermediate_size), torch.float32, dev)
+        ops.linear(h, self.w_up, u)
+        z = ops.scratch("ffn_gated", (T, self.intermediate_size), self.dtype, dev)
+        ops.activate_rows(u, z, self.activation)
+        if residual is None:
+            return ops.linear(z, self.w_down, ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev))
+        return ops.linear(z, self.w_down, residual, residual)
+
+
 register_feed_forward("swiglu", SwiGLU)
+register_feed_forward("act_mlp", ActMLP)
 register_feed_forward("gelu_glu", GeluGLU)
 register_feed_forward("clamped_glu", ClampedGLU)

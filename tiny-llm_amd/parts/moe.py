@@ -1,4 +1,6 @@
-"""A mixture of small gated feed-forward layers without a router: a table gives every token id its
+"""Mixtures of small feed-forward layers.
+
+`table_moe`: a mixture of small gated feed-forward layers without a router: a table gives every token id its
 `top` experts, each with weight 1 / top; an optional shared expert runs for every token and is added,
 optionally times sigmoid(w_sg . h), one number per token.
 
@@ -6,6 +8,12 @@ Experts are `clamped_glu` units (parts/mlp.py): down(g * sigmoid(alpha g) * (u +
 g = min(gate(h), limit), u = clamp(up(h), -limit, limit), without biases.  Their weights are stacked on
 load ([E, 2F, W] and [E, W, F]); a step multiplies every token's row with the weights of its own experts.
 Tensor names below the prefix: e<i>.gate|up|down, table, shared.gate|up|down, shared.sg.
+
+`routed_moe`: experts down(act(up(h))) without gate or bias, chosen by a router: scores s = softmax(W_router h)
+over all experts (float32); the experts lie in `groups` equal runs of neighbours, a run's score is its largest
+score and only experts of the `keep` best runs may be chosen; the `top` largest scores among those are chosen and
+weigh s_j / (sum of the chosen + 1e-20) * scale; an optional shared expert of the same form runs for every token
+and is added.  Tensor names below the prefix: e<i>.up|down, router, shared.up|down.
 """
 from __future__ import annotations
 
@@ -15,7 +23,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, WeightSpec, add_to_residual, register_feed_forward
-from .mlp import ClampedGLU
+from .mlp import ActMLP, ClampedGLU
 
 
 class TableMoE(FeedForward):
@@ -124,4 +132,104 @@ class TableMoE(FeedForward):
         return add_to_residual(residual, out)
 
 
+class RoutedMoE(FeedForward):
+    graph_safe = True
+    GROUPED_ROWS = 64       # from this many rows (tokens * top) on, a bfloat16 step groups its rows by expert
+    RUN_ROWS = 64           # from this many rows an expert on average, the rows are copied into runs of 256 an expert
+
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, num_experts: int, top: int, intermediate_size: int,
+                 groups: int = 1, keep: int = 1, scale: float = 1.0, activation: str = "relu2",
+                 shared: Optional[dict] = None):
+        """shared: None, or {"intermediate_size": F} (optionally "activation") for the shared expert."""
+        super().__init__(prefix, dtype, device)
+        self.hidden_size, self.num_experts, self.top = int(hidden_size), int(num_experts), int(top)
+        self.intermediate_size, self.scale = int(intermediate_size), float(scale)
+        self.groups, self.keep = max(1, int(groups or 1)), int(keep or 1)
+        if not (0 < self.top <= self.num_experts <= ops.MOE_MAX_ROUTED):
+            raise ValueError(f"{prefix}: 1 to {ops.MOE_MAX_ROUTED} experts and 1 to all of them a token, got "
+                             f"{self.num_experts} and top = {self.top}")
+        if self.groups > 1 and (self.num_experts % self.groups or not (0 < self.keep <= self.groups)
+                                or self.top > self.keep * (self.num_experts // self.groups)):
+            raise ValueError(f"{prefix}: {self.num_experts} experts in {self.groups} groups of which {self.keep} are "
+                             f"kept: groups must be equal and the kept ones hold at least top = {self.top} experts")
+        if activation not in ops.MOE_ACTIVATIONS or activation is None:
+            raise ValueError(f"{prefix}: activation {activation!r} is not built; known: relu2")
+        self.activation = activation
+        ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
+        ops.check_linear_sizes(dtype, self.intermediate_size, f"{prefix}: expert intermediate_size")
+        self.shared = None
+        if shared:
+            self.shared = ActMLP(f"{prefix}.shared", dtype, device, hidden_size=self.hidden_size,
+                                 intermediate_size=int(shared["intermediate_size"]),
+                                 activation=shared.get("activation", activation))
+        self.w_up = self.w_down = self.w_router = None
+
+    def weights(self) -> List[WeightSpec]:
+        p, W, F = self.prefix, self.hidden_size, self.intermediate_size
+        out = []
+        for e in range(self.num_experts):
+            out += [WeightSpec(f"{p}.e{e}.up", (F, W)), WeightSpec(f"{p}.e{e}.down", (W, F))]
+        out.append(WeightSpec(f"{p}.router", (self.num_experts, W)))
+        if self.shared is not None:
+            out += self.shared.weights()
+        return out
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        p, E = self.prefix, self.num_experts
+        self.w_up = torch.stack([tensors[f"{p}.e{e}.up"] for e in range(E)]).contiguous()
+        self.w_down = torch.stack([tensors[f"{p}.e{e}.down"] for e in range(E)]).contiguous()
+        self.w_router = tensors[f"{p}.router"].contiguous()
+        if self.shared is not None:
+            self.shared.bind(tensors)
+
+    def forward(self, h, ctx, residual):
+        T, dev, F, E, top = h.shape[0], h.device, self.intermediate_size, self.num_experts, self.top
+        # the router: logits, scores and weights in float32
+        logits = ops.scratch("moe_router", (T, E), torch.float32, dev)
+        ops.linear(h, self.w_router, logits)
+        ids = ops.scratch("moe_ids", (T, top), torch.int32, dev)
+        wts = ops.scratch("moe_weights", (T, top), torch.float32, dev)
+        ops.moe_route(logits, ids, wts, self.groups, self.keep, self.scale)
+        base = self.shared.forward(h, ctx, None) if self.shared is not None else None
+        rows = T * top
+        out = base if base is not None else ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev)
+        if self.dtype == torch.bfloat16 and rows >= self.RUN_ROWS * E:
+            # very many rows (prompts): every expert's rows side by side in runs of 256, and the tiled product of
+            # the dense layers with a weight matrix per run
+            R = ops.MOE_RUN_ROWS
+            cap = ops.moe_max_tiles(rows, E, R) * R
+            plan = ops.scratch("moe_plan", (ops.moe_plan_ints(rows, E, R),), torch.int32, dev)
+            ops.moe_plan(None, ids, plan, E, R, num_tokens=T)
+            runs = ops.moe_tile_experts(plan, rows, E, R)
+            hp = ops.scratch("moe_rows_in", (cap, self.hidden_size), self.dtype, dev)
+            pos = ops.scratch("moe_row_pos", (rows,), torch.int32, dev)
+            ops.moe_gather(h, top, plan, rows, E, R, hp, pos)
+            up = ops.scratch("moe_up", (cap, F), torch.float32, dev)        # float32: rounded once, behind the activation
+            ops.linear_grouped(hp, self.w_up, runs, up)
+            z = ops.activate_rows(up, ops.scratch("moe_gated", (cap, F), self.dtype, dev), self.activation)
+            y = ops.scratch("moe_rows_out", (cap, self.hidden_size), torch.float32, dev)
+            ops.linear_grouped(z, self.w_down, runs, y)
+            ops.moe_combine_at(y, pos, out, top, 1.0, base, None, wts)
+        elif self.dtype == torch.bfloat16 and rows >= self.GROUPED_ROWS:
+            # many rows: sorted by expert on the device, tiles of one expert's rows on the matrix cores
+            up = ops.scratch("moe_up", (rows, F), torch.float32, dev)
+            plan = ops.scratch("moe_plan", (ops.moe_plan_ints(rows, E),), torch.int32, dev)
+            ops.moe_plan(None, ids, plan, E, num_tokens=T)
+            ops.grouped_rows_gemm(h, top, self.w_up, plan, up)
+            z = ops.activate_rows(up, ops.scratch("moe_gated", (rows, F), self.dtype, dev), self.activation)
+            y = ops.scratch("moe_rows_out", (rows, self.hidden_size), torch.float32, dev)
+            ops.grouped_rows_gemm(z, 1, self.w_down, plan, y)
+            ops.moe_combine(y, out, top, 1.0, base, None, wts)
+        else:
+            # few rows (decoding) and float32: each row against its own expert's weights, the activation in
+            # the first product's kernel
+            z = ops.scratch("moe_gated", (rows, F), self.dtype, dev)
+            ops.table_moe_up(h, self.w_up, None, ids, z, self.activation)
+            ops.table_moe_down(z, self.w_down, None, ids, out, 1.0, base, None, wts)
+        if residual is None:
+            return out
+        return add_to_residual(residual, out)
+
+
 register_feed_forward("table_moe", TableMoE)
+register_feed_forward("routed_moe", RoutedMoE)
