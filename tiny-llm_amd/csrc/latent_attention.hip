@@ -260,14 +260,17 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
   const int kv_end = positions[tok0 + ntok - 1] + 1;  // what the tile's last token sees
   const int n_kt = (kv_end + 15) / 16;
   // the first key tile that the tile's first token still sees through its window
-  const int kt0 = window > 0 ? max(0, positions[tok0] - window + 1) / 16 : 0;
+  const int kv_first = window > 0 ? max(0, positions[tok0] - window + 1) : 0;
+  const int kt0 = kv_first / 16;
   const int lowest = window > 0 ? pos - window : -1;  // keys at or before this position are hidden from this row
   const float c_log2 = scale * 1.44269504088896f;
   __syncthreads();
 
   bf16x8 kop[LF_MAXKS];
   auto fetch = [&](int kt) {
-    const int j = min(kt * 16 + c, kv_end - 1);       // keys beyond the end read a row that exists
+    // keys beyond the end, and keys that every window of the tile has left (their pages may have been given
+    // back), read a row that exists: they are masked, but what they hold would still enter the products
+    const int j = max(min(kt * 16 + c, kv_end - 1), kv_first);
     const int64_t slot = (int64_t)bt[j / block_size] * block_size + (j % block_size);
 #pragma unroll
     for (int ks = 0; ks < LF_MAXKS; ++ks) {
@@ -470,7 +473,8 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_prefill_bf16_kernel
 #pragma unroll
     for (int j = 0; j < LP_NPF; ++j) {
       const int f = tid + j * LF_WAVES * TL_WAVE;
-      const int key = min(kt * LP_KEYS + min(f / CPR, LP_KEYS - 1), kv_end - 1);     // keys beyond the end read a row that exists
+      // keys beyond the end, and keys every window has left (their pages may be given back), read a row that exists
+      const int key = max(min(kt * LP_KEYS + min(f / CPR, LP_KEYS - 1), kv_end - 1), kv_first);
       page[j] = bt[key / block_size];
     }
   };
@@ -480,7 +484,7 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_prefill_bf16_kernel
       const int f = tid + j * LF_WAVES * TL_WAVE;
       if (f < LP_KEYS * CPR) {
         const int row = f / CPR, d0 = (f - row * CPR) * 8;
-        const int key = min(kt * LP_KEYS + row, kv_end - 1);
+        const int key = max(min(kt * LP_KEYS + row, kv_end - 1), kv_first);
         const int64_t slot = (int64_t)page[j] * block_size + (key % block_size);
         if (d0 < kv_rank) pf[j] = *(const bf16x8*)(latent + slot * kv_rank + d0);
         else if (d0 - kv_rank < rot) pf[j] = *(const bf16x8*)(rope + slot * rot + (d0 - kv_rank));
