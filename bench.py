@@ -13,7 +13,7 @@ Llama-3-8B shape; 64 requests of 1,024 tokens that nearly fill the cache at the 
 `--only` picks a part (for profiling), or one of the measurements that are not part of the line:
 `attention` (the attention kernels alone at contexts up to 131,072 tokens), `long_context` (the Llama-3-8B
 shape with 8 requests of 32,000 tokens and one of 131,000), `decode_shapes` (decode steps at the two larger
-shapes by batch), `host` (a step's wall time against its time on the GPU), `fofapel` (the Fofapel design, as `lufazen`), `lufazen` (the Lufazen design,
+shapes by batch), `host` (a step's wall time against its time on the GPU), `gesutar` and `fofapel` (those designs, as `lufazen`), `lufazen` (the Lufazen design,
 recurrent and latent-attention layers, at two sizes beside a Llama of equal size: prefill, decode, time by kernel).
 """
 import argparse
@@ -732,7 +732,7 @@ def kernels_by_name(run):
         run()
         torch.cuda.synchronize()
     evs = [e for e in prof.events() if e.device_type == DeviceType.CUDA and "emcpy" not in e.name and "emset" not in e.name]
-    steps = max(1, sum(1 for e in evs if "embedding_kernel" in e.name))
+    steps = max(1, sum(1 for e in evs if "embedding_kernel" in e.name or "embedding_pairs_kernel" in e.name))
     out = {}
     import re
     for e in evs:
@@ -813,6 +813,43 @@ def fofapel_figures(args):
     return design_beside_llama(args, "fofapel", fofapel_config, bounds)
 
 
+def gesutar_config(layers, width, ff, heads, vocab=32000, window=512):
+    """Every layer: attention over cached latents of 512 in a window of 512 tokens (128 unrotated + 64 rotated
+    query/key dims, values of 128, a sink per head, a gate per element) and 16 routed experts of ff / 8 in four
+    groups of which two are kept, four a token, beside a shared expert of ff / 4 (three quarters of a dense
+    layer's hidden units a token); the embedding with a pair table of 65,521 buckets."""
+    out = []
+    for _ in range(layers):
+        mixer = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "mask": {"size": window},
+                 "rot": {"base": 10000.0, "dims": 64}, "scale": 192 ** -0.5}
+        mlp = {"kind": "moe", "router": {"experts": 16, "top": 4, "scale": 1.0, "groups": {"count": 4, "keep": 2}},
+               "expert": {"ff": ff // 8}, "shared": {"ff": ff // 4}}
+        out.append({"type": "latent_attention", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Gesutar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}},
+            "layers": out, "max_position": 8192}
+
+
+def gesutar_figures(args):
+    """The Gesutar design at two sizes beside a Llama of equal layers, width, feed-forward size, heads of 128 and
+    vocabulary, as `lufazen_figures`; bounds for the kernels that only this design has."""
+    def bounds(dtype, heads, width, ff):
+        e = ELT[dtype]
+        T, ctx, B, win = PREFILL_TOKENS, PROMPT_LEN, 8, 512
+        kr, rot = 512, 64
+        return {
+            "latent attention prefill (flops of scores and values over the latent inside the window)":
+                round(2.0 * heads * T * min(win, T / 2) * (2 * kr + rot) / (PEAK_TFLOPS[dtype] * 1e12) * 1e6, 1),
+            "latent attention decode b8 (the cached latents of the window once)":
+                round(B * min(ctx, win) * (kr + rot) * e / (HBM_GBS * 1e9) * 1e6, 2),
+            "experts decode b8 (the weights of all 16 experts once)":
+                round(16 * 2 * width * (ff // 8) * e / (HBM_GBS * 1e9) * 1e6, 2),
+            "experts prefill (flops of four experts a token)":
+                round(2.0 * T * 4 * 2 * width * (ff // 8) / (PEAK_TFLOPS[dtype] * 1e12) * 1e6, 1),
+        }
+    return design_beside_llama(args, "gesutar", gesutar_config, bounds)
+
+
 def design_beside_llama(args, design, config_of, bounds_of):
     import torch
     dtype = args.dtype
@@ -866,6 +903,9 @@ def run(args):
         return
     if args.only == "fofapel":
         print(json.dumps({"fofapel_beside_llama": fofapel_figures(args)}), flush=True)
+        return
+    if args.only == "gesutar":
+        print(json.dumps({"gesutar_beside_llama": gesutar_figures(args)}), flush=True)
         return
     if args.only == "attention":
         print(json.dumps({"decode_attention": attention_sweep()}), flush=True)
@@ -942,7 +982,7 @@ def main():
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--only", default="all",
                     choices=["all", "headline", "decode", "prefill", "fp32", "kernels", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host",
-                             "attention", "long_context", "decode_shapes", "lufazen", "fofapel"],
+                             "attention", "long_context", "decode_shapes", "lufazen", "fofapel", "gesutar"],
                     help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
                          "one of them (profiling); fp32: the float32 figures as the headline; kernels: decode with the time of "
                          "a step by kernel (torch's profiler); peaks / llama3_8b / "
@@ -950,7 +990,7 @@ def main():
                          "attention kernels alone at contexts up to 131,072 tokens; long_context: the Llama-3-8B shape with "
                          "8 requests of 32,000 tokens and one of 131,000; decode_shapes: decode steps at the two larger shapes by batch; "
                          "lufazen: prefill and decode of the Lufazen design at two sizes beside a Llama of equal size, by kernel; "
-                         "fofapel: the same for the Fofapel design")
+                         "fofapel, gesutar: the same for the Fofapel and the Gesutar design")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         if int(os.environ.get("RANK", "0")) == 0:

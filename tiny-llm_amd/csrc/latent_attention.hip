@@ -663,7 +663,8 @@ __global__ __launch_bounds__(kThreads) void head_products_kernel(const TI* __res
                                                                  int in_head_width, const TW* __restrict__ w,
                                                                  TO* __restrict__ out, int64_t out_stride,
                                                                  int out_head_width, int n_rows, int inner, int cols,
-                                                                 int cols_padded) {
+                                                                 int cols_padded, const TI* __restrict__ gate,
+                                                                 int64_t gate_stride) {
   __shared__ float xs[kRows][kMaxInner];
   __shared__ float part[kWaves][kRows][kHpCols];
   const int h = blockIdx.x, wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
@@ -734,7 +735,11 @@ __global__ __launch_bounds__(kThreads) void head_products_kernel(const TI* __res
     float sum = 0.f;
 #pragma unroll
     for (int q = 0; q < kWaves; ++q) sum += part[q][r][c2];
-    if (n2 < cols) out[(int64_t)(t0 + r) * out_stride + (int64_t)h * out_head_width + n2] = from_f32<TO>(sum);
+    if (n2 < cols) {
+      // a gate per element (optional): its pre-activations lie as the heads' results do, cols a head
+      if (gate) sum /= 1.f + expf(-to_f32(gate[(int64_t)(t0 + r) * gate_stride + (int64_t)h * cols + n2]));
+      out[(int64_t)(t0 + r) * out_stride + (int64_t)h * out_head_width + n2] = from_f32<TO>(sum);
+    }
   }
 }
 
@@ -748,7 +753,8 @@ template <typename TO>
 __global__ __launch_bounds__(kThreads) void head_gemm_bf16_kernel(const bf16_t* __restrict__ in, int64_t in_stride,
                                                                   int in_head_width, const bf16_t* __restrict__ w,
                                                                   TO* __restrict__ out, int64_t out_stride,
-                                                                  int out_head_width, int n_rows, int inner, int cols) {
+                                                                  int out_head_width, int n_rows, int inner, int cols,
+                                                                  const bf16_t* __restrict__ gate, int64_t gate_stride) {
   const int h = blockIdx.x, wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE, g = lane / 16, c = lane % 16;
   const int col0 = blockIdx.y * 64 + (wave & 1) * 32, row0 = blockIdx.z * 64 + (wave >> 1) * 32;
   if (col0 >= cols || row0 >= n_rows) return;
@@ -789,7 +795,11 @@ __global__ __launch_bounds__(kThreads) void head_gemm_bf16_kernel(const bf16_t* 
       TO* dst = out + (int64_t)row * out_stride + (int64_t)h * out_head_width + n;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (n + i < cols) dst[i] = from_f32<TO>(acc[a][b][i]);
+        if (n + i < cols) {
+          float v = acc[a][b][i];
+          if (gate) v /= 1.f + expf(-(float)gate[(int64_t)row * gate_stride + (int64_t)h * cols + n + i]);
+          dst[i] = from_f32<TO>(v);
+        }
     }
   }
 }
@@ -924,10 +934,12 @@ int tl_latent_prefill(const float* qa, const void* latent, const void* rope, con
 }
 
 // in / out: rows with a stride, head h at column h * head_width.  w [heads, inner, cols_padded] of in's type;
-// out float32 (out_dtype 0) or of in's type.
+// out float32 (out_dtype 0) or of in's type.  gate (optional, of in's type): rows of heads * cols pre-activations
+// with a stride; the result is multiplied by their sigmoid, element by element.
 int tl_head_products(const void* in, int64_t in_stride, int in_head_width, const void* w, void* out,
                      int64_t out_stride, int out_head_width, int n_rows, int heads, int inner, int cols,
-                     int cols_padded, int dtype, int out_dtype, hipStream_t stream) {
+                     int cols_padded, const void* gate, int64_t gate_stride, int dtype, int out_dtype,
+                     hipStream_t stream) {
   if (n_rows <= 0) return TL_OK;
   if (heads <= 0 || inner <= 0 || inner > kMaxInner || cols <= 0 || inner > in_head_width || cols > out_head_width ||
       cols_padded < cols || cols_padded % 8 ||
@@ -936,7 +948,8 @@ int tl_head_products(const void* in, int64_t in_stride, int in_head_width, const
   dim3 g(heads, (cols + kHpCols - 1) / kHpCols, (n_rows + kRows - 1) / kRows), b(kThreads);
 #define TL_HP(TI, TO)                                                                                              \
   hipLaunchKernelGGL((head_products_kernel<TI, TI, TO>), g, b, 0, stream, (const TI*)in, in_stride, in_head_width, \
-                     (const TI*)w, (TO*)out, out_stride, out_head_width, n_rows, inner, cols, cols_padded)
+                     (const TI*)w, (TO*)out, out_stride, out_head_width, n_rows, inner, cols, cols_padded,         \
+                     (const TI*)gate, gate_stride)
   if (dtype == 0 && out_dtype == 0) TL_HP(float, float);
   else if (dtype == 1 && out_dtype == 0) TL_HP(bf16_t, float);
   else if (dtype == 1 && out_dtype == 1) TL_HP(bf16_t, bf16_t);
@@ -947,7 +960,8 @@ int tl_head_products(const void* in, int64_t in_stride, int in_head_width, const
 
 // bfloat16, many rows: w [heads, cols, inner]; inner a multiple of 8, operands 16-byte aligned.
 int tl_head_gemm(const void* in, int64_t in_stride, int in_head_width, const void* w, void* out, int64_t out_stride,
-                 int out_head_width, int n_rows, int heads, int inner, int cols, int out_dtype, hipStream_t stream) {
+                 int out_head_width, int n_rows, int heads, int inner, int cols, const void* gate, int64_t gate_stride,
+                 int out_dtype, hipStream_t stream) {
   if (n_rows <= 0) return TL_OK;
   if (heads <= 0 || inner <= 0 || inner % 8 || cols <= 0 || inner > in_head_width || cols > out_head_width ||
       in_stride % 8 || in_head_width % 8 || (n_rows + 63) / 64 > 65535 || (cols + 63) / 64 > 65535)
@@ -955,10 +969,12 @@ int tl_head_gemm(const void* in, int64_t in_stride, int in_head_width, const voi
   dim3 g(heads, (cols + 63) / 64, (n_rows + 63) / 64), b(kThreads);
   if (out_dtype == 0)
     hipLaunchKernelGGL(head_gemm_bf16_kernel<float>, g, b, 0, stream, (const bf16_t*)in, in_stride, in_head_width,
-                       (const bf16_t*)w, (float*)out, out_stride, out_head_width, n_rows, inner, cols);
+                       (const bf16_t*)w, (float*)out, out_stride, out_head_width, n_rows, inner, cols,
+                       (const bf16_t*)gate, gate_stride);
   else if (out_dtype == 1)
     hipLaunchKernelGGL(head_gemm_bf16_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)in, in_stride, in_head_width,
-                       (const bf16_t*)w, (bf16_t*)out, out_stride, out_head_width, n_rows, inner, cols);
+                       (const bf16_t*)w, (bf16_t*)out, out_stride, out_head_width, n_rows, inner, cols,
+                       (const bf16_t*)gate, gate_stride);
   else
     return TL_ERR_ARG;
   return tl_launch_status();

@@ -1365,14 +1365,23 @@ def head_product_weights(w: torch.Tensor) -> torch.Tensor:
     return torch.nn.functional.pad(w, (0, pad)).contiguous() if pad else w.contiguous()
 
 
-def head_products(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def _head_gate(gate: Optional[torch.Tensor], x: torch.Tensor, T: int, H: int, cols: int, what: str):
+    if gate is not None:
+        _dev(gate)
+        _need(gate.dim() == 2 and gate.stride(1) == 1 and tuple(gate.shape) == (T, H * cols) and gate.dtype == x.dtype,
+              f"{what}: the gate is [T, heads * cols] of the input's type (rows may be wider apart)")
+
+
+def head_products(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t, h, :] = w[h]^T x[t, h, :] for every head in one launch (steps of few rows):
     x [T, heads, >= inner] and out [T, heads, >= cols] may be views into wider rows (any row and
     head stride, unit inner stride); w [heads, inner, cols rounded up to 8] from `head_product_weights`,
-    of x's type; out float32 or x's type (its last size says how many columns are real)."""
+    of x's type; out float32 or x's type (its last size says how many columns are real).  gate [T, heads * cols]
+    (optional, x's type): out is multiplied by sigmoid(gate) element by element."""
     _dev(x, w, out)
     T, H = x.shape[0], x.shape[1]
     inner, cols = w.shape[1], out.shape[2]
+    _head_gate(gate, x, T, H, cols, "head_products")
     if not (x.dim() == 3 and out.dim() == 3 and w.dim() == 3 and w.is_contiguous() and w.shape[0] == H
             and w.dtype == x.dtype and x.stride(2) == 1 and out.stride(2) == 1 and tuple(out.shape[:2]) == (T, H)
             and x.shape[2] == inner and w.shape[2] % 8 == 0 and 0 <= w.shape[2] - cols < 8
@@ -1380,18 +1389,20 @@ def head_products(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.
         _fail("head_products: x [T, heads, inner], w [heads, inner, cols rounded up to 8], out [T, heads, cols]")
     _check(_lib().tl_head_products(_ptr(x), c_int64(x.stride(0)), c_int(x.stride(1)), _ptr(w, 16), _ptr(out),
                                    c_int64(out.stride(0)), c_int(out.stride(1)), c_int(T), c_int(H), c_int(inner),
-                                   c_int(cols), c_int(w.shape[2]), c_int(_dt(x)), c_int(_dt(out)), _stream()),
-           "head_products")
+                                   c_int(cols), c_int(w.shape[2]), _ptr(gate),
+                                   c_int64(gate.stride(0) if gate is not None else 0), c_int(_dt(x)), c_int(_dt(out)),
+                                   _stream()), "head_products")
     return out
 
 
-def head_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def head_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t, h, :] = w[h] x[t, h, :] for every head in one launch on the matrix cores (bfloat16, any
     number of rows): x [T, heads, inner] and out [T, heads, cols] may be views into wider rows; w
-    [heads, cols, inner] contiguous; out bfloat16 or float32."""
+    [heads, cols, inner] contiguous; out bfloat16 or float32.  gate: as in `head_products`."""
     _dev(x, w, out)
     T, H = x.shape[0], x.shape[1]
     cols, inner = w.shape[1], w.shape[2]
+    _head_gate(gate, x, T, H, cols, "head_gemm")
     if not (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 3 and out.dim() == 3 and w.dim() == 3
             and w.is_contiguous() and w.shape[0] == H and x.stride(2) == 1 and out.stride(2) == 1
             and tuple(out.shape[:2]) == (T, H) and x.shape[2] == inner and out.shape[2] == cols and inner % 8 == 0
@@ -1399,7 +1410,8 @@ def head_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tens
         _fail("head_gemm: bfloat16 x [T, heads, inner] (inner and strides multiples of 8), w [heads, cols, inner], out [T, heads, cols]")
     _check(_lib().tl_head_gemm(_ptr(x, 16), c_int64(x.stride(0)), c_int(x.stride(1)), _ptr(w, 16), _ptr(out),
                                c_int64(out.stride(0)), c_int(out.stride(1)), c_int(T), c_int(H), c_int(inner),
-                               c_int(cols), c_int(_dt(out)), _stream()), "head_gemm")
+                               c_int(cols), _ptr(gate), c_int64(gate.stride(0) if gate is not None else 0),
+                               c_int(_dt(out)), _stream()), "head_gemm")
     return out
 
 

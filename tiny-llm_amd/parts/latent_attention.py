@@ -215,15 +215,16 @@ class LatentAttention(Mixer):
         T, H, KR = mix.shape
         V, dev = self.value_dim, mix.device
         o = ops.scratch("latent_heads", (T, H * V), self.dtype, dev)
+        gate = down[:, self.g_off:self.g_off + H * V] if self.gate == "element" else None
         if few:
-            ops.head_products(mix, self.w_uv_few, o.view(T, H, V))
+            ops.head_products(mix, self.w_uv_few, o.view(T, H, V), gate)      # the gate rides in the product
         elif many:
-            ops.head_gemm(mix, self.w_uv.view(H, V, KR), o.view(T, H, V))
+            ops.head_gemm(mix, self.w_uv.view(H, V, KR), o.view(T, H, V), gate)
         else:
             for n in range(H):
                 ops.linear(mix[:, n, :], self.w_uv[n * V:(n + 1) * V], o[:, n * V:(n + 1) * V])
-        if self.gate == "element":
-            ops.gate_rows(o, down[:, self.g_off:self.g_off + H * V], o)
+            if gate is not None:
+                ops.gate_rows(o, gate, o)
         if residual is None:
             return ops.linear(o, self.w_o, ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev))
         return ops.linear(o, self.w_o, residual, residual)

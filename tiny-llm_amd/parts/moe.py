@@ -181,16 +181,38 @@ class RoutedMoE(FeedForward):
         self.w_router = tensors[f"{p}.router"].contiguous()
         if self.shared is not None:
             self.shared.bind(tensors)
+            # one product reads h for the router's logits and the shared expert's hidden units (float32 out):
+            # [router, its rows filled up to a multiple of 8 | shared up]
+            self.shared_off = -(-E // 8) * 8
+            first = torch.zeros((self.shared_off + self.shared.intermediate_size, self.hidden_size), dtype=self.dtype,
+                                device=self.w_router.device)
+            first[:E] = self.w_router
+            first[self.shared_off:] = self.shared.w_up
+            self.w_first = first
 
     def forward(self, h, ctx, residual):
         T, dev, F, E, top = h.shape[0], h.device, self.intermediate_size, self.num_experts, self.top
         # the router: logits, scores and weights in float32
-        logits = ops.scratch("moe_router", (T, E), torch.float32, dev)
-        ops.linear(h, self.w_router, logits)
         ids = ops.scratch("moe_ids", (T, top), torch.int32, dev)
         wts = ops.scratch("moe_weights", (T, top), torch.float32, dev)
-        ops.moe_route(logits, ids, wts, self.groups, self.keep, self.scale)
-        base = self.shared.forward(h, ctx, None) if self.shared is not None else None
+        if self.shared is not None:
+            # with the shared expert's first product; its second one writes the sum the experts are added to
+            # (the residual stream itself where the caller gives it)
+            Fs = self.shared.intermediate_size
+            first = ops.scratch("moe_first", (T, self.shared_off + Fs), torch.float32, dev)
+            ops.linear(h, self.w_first, first)
+            ops.moe_route(first[:, :E], ids, wts, self.groups, self.keep, self.scale)
+            zs = ops.activate_rows(first[:, self.shared_off:], ops.scratch("ffn_gated", (T, Fs), self.dtype, dev),
+                                   self.shared.activation)
+            if residual is None:
+                base = ops.linear(zs, self.shared.w_down, ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev))
+            else:
+                base = ops.linear(zs, self.shared.w_down, residual, residual)
+        else:
+            logits = ops.scratch("moe_router", (T, E), torch.float32, dev)
+            ops.linear(h, self.w_router, logits)
+            ops.moe_route(logits, ids, wts, self.groups, self.keep, self.scale)
+            base = residual                     # the experts are added to the stream itself (or stand alone)
         rows = T * top
         out = base if base is not None else ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev)
         if self.dtype == torch.bfloat16 and rows >= self.RUN_ROWS * E:
@@ -226,9 +248,7 @@ class RoutedMoE(FeedForward):
             z = ops.scratch("moe_gated", (rows, F), self.dtype, dev)
             ops.table_moe_up(h, self.w_up, None, ids, z, self.activation)
             ops.table_moe_down(z, self.w_down, None, ids, out, 1.0, base, None, wts)
-        if residual is None:
-            return out
-        return add_to_residual(residual, out)
+        return out
 
 
 register_feed_forward("table_moe", TableMoE)
