@@ -194,11 +194,20 @@ __global__ __launch_bounds__(TL_WAVE) void row_dot_sigmoid_kernel(const T* __res
 // order inside an expert is whatever the atomics give: a row's result does not depend on its place).
 constexpr int kTileRows = 32;
 
-__global__ void moe_count_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ table,
-                                 int32_t* __restrict__ counts, int rows, int top, int experts, int vocab) {
+// A workgroup counts its 256 rows in LDS first and adds one number per expert to the shared counters (a prompt's
+// thousands of rows over a few experts would otherwise queue up at a handful of addresses).
+__global__ __launch_bounds__(kThreads) void moe_count_kernel(const int32_t* __restrict__ tokens,
+                                                             const int32_t* __restrict__ table,
+                                                             int32_t* __restrict__ counts, int rows, int top,
+                                                             int experts, int vocab) {
+  __shared__ int32_t local[1024];
+  for (int e = threadIdx.x; e < experts; e += kThreads) local[e] = 0;
+  __syncthreads();
   const int i = blockIdx.x * kThreads + threadIdx.x;
-  if (i >= rows) return;
-  atomicAdd(&counts[expert_of(tokens, table, i / top, i % top, top, vocab, experts)], 1);
+  if (i < rows) atomicAdd(&local[expert_of(tokens, table, i / top, i % top, top, vocab, experts)], 1);
+  __syncthreads();
+  for (int e = threadIdx.x; e < experts; e += kThreads)
+    if (local[e]) atomicAdd(&counts[e], local[e]);
 }
 
 // One workgroup: offsets of the experts' runs in `sorted`, and the list of tiles.
@@ -277,13 +286,27 @@ __global__ void moe_combine_at_kernel(const float* __restrict__ y, const int32_t
   out[i] = fmaf(coef, acc, b);
 }
 
-__global__ void moe_scatter_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ table,
-                                   const int32_t* __restrict__ offsets, int32_t* __restrict__ cursor,
-                                   int32_t* __restrict__ sorted, int rows, int top, int experts, int vocab) {
+// A workgroup ranks its rows inside every expert in LDS, takes one range per expert from the shared cursors and
+// writes its rows there.
+__global__ __launch_bounds__(kThreads) void moe_scatter_kernel(const int32_t* __restrict__ tokens,
+                                                               const int32_t* __restrict__ table,
+                                                               const int32_t* __restrict__ offsets,
+                                                               int32_t* __restrict__ cursor, int32_t* __restrict__ sorted,
+                                                               int rows, int top, int experts, int vocab) {
+  __shared__ int32_t local[1024];
+  for (int e = threadIdx.x; e < experts; e += kThreads) local[e] = 0;
+  __syncthreads();
   const int i = blockIdx.x * kThreads + threadIdx.x;
-  if (i >= rows) return;
-  const int e = expert_of(tokens, table, i / top, i % top, top, vocab, experts);
-  sorted[offsets[e] + atomicAdd(&cursor[e], 1)] = i;
+  int e = 0, rank = 0;
+  if (i < rows) {
+    e = expert_of(tokens, table, i / top, i % top, top, vocab, experts);
+    rank = atomicAdd(&local[e], 1);
+  }
+  __syncthreads();
+  for (int x = threadIdx.x; x < experts; x += kThreads)       // the count turns into the range's first place
+    if (local[x]) local[x] = offsets[x] + atomicAdd(&cursor[x], local[x]);
+  __syncthreads();
+  if (i < rows) sorted[local[e] + rank] = i;
 }
 
 // out[row, n] = sum_k a[row / a_div, k] * w[expert of row][n, k] for the rows of one tile; bfloat16 operands

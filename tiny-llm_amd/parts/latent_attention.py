@@ -32,6 +32,7 @@ import torch
 
 from ..kernels import ops
 from .base import CacheSpec, CacheTensor, LayerCache, Mixer, POSITION_ENCODINGS, WeightSpec, register_mixer
+from .norm import LazyNorm
 
 
 def _pad8(n: int) -> int:
@@ -40,6 +41,7 @@ def _pad8(n: int) -> int:
 
 class LatentAttention(Mixer):
     graph_safe = True
+    accepts_lazy_norm = True        # a pre-norm block's norm rides in the one product that reads h
 
     def __init__(self, prefix, dtype, device, *, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int,
                  value_dim: int, q_rank: int, kv_rank: int, scale: float, eps: float, position: dict = None,
@@ -150,13 +152,17 @@ class LatentAttention(Mixer):
         if cache.write == self.shares_cache:
             raise ValueError(f"{self.prefix}: a layer with a down projection of its own writes its cache, "
                              "one without reads another layer's")
-        T, dev, H = h.shape[0], h.device, self.num_heads
+        lazy = h if isinstance(h, LazyNorm) else None
+        T, dev, H = (lazy.num_rows, lazy.x.device, self.num_heads) if lazy is not None else (h.shape[0], h.device, self.num_heads)
         R, D, V, KR = self.rot_dim, self.head_dim, self.value_dim, self.kv_rank
         tables = self.position.rotary_tables()
         cos, sin = (tables[0], tables[1]) if tables is not None else (None, None)
         latent, rope = cache.tensors["latent"], cache.tensors.get("rope_key")
         down = ops.scratch("latent_down", (T, self.down_width), self.dtype, dev)
-        ops.linear(h, self.w_down, down)
+        if lazy is not None:
+            lazy.linear(self.w_down, down)
+        else:
+            ops.linear(h, self.w_down, down)
         kv = () if self.shares_cache else (self.kv_off, KR, R, self.rdims, self.w_dkv_norm, ctx.positions, cos, sin,
                                            ctx.slot_mappings[cache.group], latent, rope, self.pairing)
         if self.q_rank:
