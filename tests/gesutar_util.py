@@ -37,9 +37,10 @@ def layer(m, mlp):
 
 
 def model(width, vocab, layers, bigram=(97, 7, 13), scale=3.0, eps=1e-5):
-    return {"architecture": "Gesutar", "vocab": vocab, "width": width, "norm": {"eps": eps},
-            "embedding": {"scale": scale, "bigram": {"buckets": bigram[0], "mul_prev": bigram[1], "mul_cur": bigram[2]}},
-            "layers": layers}
+    emb = {"scale": scale}
+    if bigram:
+        emb["bigram"] = {"buckets": bigram[0], "mul_prev": bigram[1], "mul_cur": bigram[2]}
+    return {"architecture": "Gesutar", "vocab": vocab, "width": width, "norm": {"eps": eps}, "embedding": emb, "layers": layers}
 
 
 # windows, head shapes, latents and rotated dims that differ from layer to layer (four cache groups); fewer
@@ -71,8 +72,11 @@ ODD = model(50, 199, [
 
 ONLY_ATTENTION = model(64, 199, [layer(mixer(6, 16, 16, 8, 64, 20, 16), None)], bigram=(50, 3, 5))
 ONLY_MOE = model(64, 199, [layer(mixer(2, 8, 8, 8, 16, 9, 8), moe(8, 3, 16, (4, 2), 2.0, 24))], bigram=(11, 2, 9))
+# no pair table: the token rows times the scale alone
+NO_PAIRS = model(64, 150, [layer(mixer(2, 16, 8, 16, 32, 12, 8), moe(3, 2, 8))], bigram=None, scale=2.0)
 
-CONFIGS = {"A": (MIX_A, 16), "B": (MIX_B, 8), "odd": (ODD, 4), "attention": (ONLY_ATTENTION, 4), "moe": (ONLY_MOE, 16)}
+CONFIGS = {"A": (MIX_A, 16), "B": (MIX_B, 8), "odd": (ODD, 4), "attention": (ONLY_ATTENTION, 4), "moe": (ONLY_MOE, 16),
+           "no_pairs": (NO_PAIRS, 8)}
 
 
 def every_expert(cfg):
@@ -135,7 +139,8 @@ def random_weights(cfg, seed=0, sharpen=3.0):
         out[name] = mean + std * rng.standard_normal(n)
 
     mat("embed", V, W, gain=np.sqrt(W) / max(cfg["embedding"].get("scale", 1.0), 1.0))
-    out["bigram"] = 0.7 * rng.standard_normal((cfg["embedding"]["bigram"]["buckets"] + 1, W))
+    if cfg["embedding"].get("bigram"):
+        out["bigram"] = 0.7 * rng.standard_normal((cfg["embedding"]["bigram"]["buckets"] + 1, W))
     for i, l in enumerate(cfg["layers"]):
         p, a = f"l{i}.", l["mixer"]
         H, D, R, Vd, C = a["heads"], a["dim"], a["rot_dim"], a["vdim"], a["kv_rank"]

@@ -42,6 +42,15 @@ def test_spec_names_the_checkpoints_tensors(name):
     assert got == want
 
 
+def test_without_a_pair_table_and_without_a_feed_forward():
+    from gesutar_util import NO_PAIRS
+    typed, spec, dec = _decoder(NO_PAIRS)
+    assert typed.bigram is None and spec.embedding.kind == "token_embedding" and dec.embedding.scale == 2.0
+    assert dec.state_specs() == {}
+    _, spec_a, _ = _decoder(MIX_A)
+    assert spec_a.ignorable_tensors == ("l2.norm2",) and "ffn" not in spec_a.layers[2].parts
+
+
 def test_cache_groups_windows_and_state():
     from tiny_llm_amd.cache import CacheManager
     _, _, dec = _decoder(MIX_A)

@@ -27,7 +27,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # off by one, a sink left out, a wrong previous token) moves a row by its whole size in either precision.
 TOL = {"float32": 2e-4, "bfloat16": 1e-1}
 LENGTHS = {"A": [70, 133, 33, 200, 97, 64], "B": [1, 9, 40, 100, 150, 57], "odd": [31, 2, 77, 50],
-           "attention": [40, 75, 130, 9], "moe": [24, 121, 48, 5]}
+           "attention": [40, 75, 130, 9], "moe": [24, 121, 48, 5], "no_pairs": [30, 3, 66]}
 
 _cache = {}
 
@@ -103,7 +103,7 @@ def all_free(runner):
         runner.cache.free_slots == runner.cache.max_seqs
 
 
-CASES = [(n, "float32") for n in ("attention", "moe", "A", "B", "odd")] + \
+CASES = [(n, "float32") for n in ("attention", "moe", "A", "B", "odd", "no_pairs")] + \
         [(n, "bfloat16") for n in ("attention", "moe", "A", "B")]
 
 

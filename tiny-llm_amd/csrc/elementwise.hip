@@ -16,7 +16,7 @@ constexpr int kWaves = kThreads / TL_WAVE;
 // ------------------------------------------------------------------ embedding
 template <typename T>
 __global__ void embedding_kernel(const int32_t* __restrict__ tokens, const T* __restrict__ table,
-                                 float* __restrict__ out, int hidden, int vocab) {
+                                 float* __restrict__ out, int hidden, int vocab, float scale) {
   const int t = blockIdx.x;
   const int tok = tokens[t];
   float* dst = out + (int64_t)t * hidden;
@@ -25,7 +25,7 @@ __global__ void embedding_kernel(const int32_t* __restrict__ tokens, const T* __
     return;
   }
   const T* src = table + (int64_t)tok * hidden;
-  for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = to_f32(src[j]);
+  for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = to_f32(src[j]) * scale;     // (times 1 is exact)
 }
 
 // out[t, :] = table[tokens[t], :] * scale + pairs[row(t), :]: a second table indexed by a hash of (the token
@@ -321,11 +321,11 @@ __global__ void decode_advance_kernel(const AdvanceArgs a) {
 extern "C" {
 
 int tl_embedding(const int32_t* tokens, const void* table, float* out, int n_tokens, int hidden,
-                 int vocab, int dtype, hipStream_t stream) {
+                 int vocab, float scale, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (hidden <= 0 || vocab <= 0) return TL_ERR_ARG;
   TL_DISPATCH_T(dtype, hipLaunchKernelGGL(embedding_kernel<T>, dim3(n_tokens), dim3(kThreads), 0, stream,
-                                          tokens, (const T*)table, out, hidden, vocab);)
+                                          tokens, (const T*)table, out, hidden, vocab, scale);)
   return tl_launch_status();
 }
 

@@ -182,8 +182,8 @@ def check_attention_sizes(dtype: torch.dtype, num_heads: int, num_kv_heads: int,
 
 
 # --------------------------------------------------------------------------- ops
-def embedding(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t, :] = table[tokens[t], :] as float32."""
+def embedding(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[t, :] = table[tokens[t], :] * scale as float32."""
     _dev(tokens, table, out)
     T = tokens.numel()
     V, H = table.shape
@@ -193,7 +193,7 @@ def embedding(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> t
         _fail("embedding table must be contiguous")
     if not (out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H)):
         _fail(f"embedding output must be float32 [{T}, {H}]")
-    _check(_lib().tl_embedding(_ptr(tokens), _ptr(table), _ptr(out), c_int(T), c_int(H), c_int(V),
+    _check(_lib().tl_embedding(_ptr(tokens), _ptr(table), _ptr(out), c_int(T), c_int(H), c_int(V), c_float(scale),
                                c_int(_dt(table)), _stream()), "embedding")
     return out
 

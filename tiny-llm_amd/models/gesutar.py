@@ -12,7 +12,6 @@ of the form down(relu(up h)^2), chosen through groups, plus a shared expert ("ro
 from __future__ import annotations
 
 from ..config.gesutar import GesutarConfig
-from ..config.llama import ConfigError
 from ..config.registry import register_architecture
 from ..config.spec import LayerSpec, ModelSpec, PartSpec, PlanEntry
 
@@ -50,10 +49,8 @@ def build_gesutar_spec(cfg: GesutarConfig) -> ModelSpec:
         embedding = PartSpec("pair_embedding", dict(sizes, buckets=cfg.bigram.buckets, mul_prev=cfg.bigram.mul_prev,
                                                     mul_cur=cfg.bigram.mul_cur, scale=cfg.embedding_scale,
                                                     pairs_name="bigram"), "embed")
-    elif cfg.embedding_scale == 1.0:
-        embedding = PartSpec("token_embedding", sizes, "embed")
     else:
-        raise ConfigError("a scaled embedding without the bigram table is not built")
+        embedding = PartSpec("token_embedding", dict(sizes, scale=cfg.embedding_scale), "embed")
     return ModelSpec(
         architecture="Gesutar",
         vocab_size=cfg.vocab,
@@ -65,6 +62,8 @@ def build_gesutar_spec(cfg: GesutarConfig) -> ModelSpec:
         final_norm=norm.named("final.norm"),
         lm_head=PartSpec("lm_head", sizes, "head"),
         eos_token_ids=cfg.eos_token_ids,
+        # a layer without feed-forward has no use for a second norm, should a checkpoint carry one
+        ignorable_tensors=tuple(f"l{i}.norm2" for i, layer in enumerate(cfg.layers) if layer.mlp is None),
     )
 
 

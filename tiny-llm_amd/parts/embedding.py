@@ -16,9 +16,11 @@ from .norm import LazyNorm
 class TokenEmbedding(Embedding):
     graph_safe = True
 
-    def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int, weight_name: str = "weight"):
+    def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int, weight_name: str = "weight",
+                 scale: float = 1.0):
+        """scale: a constant the rows are multiplied by (in float32)."""
         super().__init__(prefix, dtype, device)
-        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.vocab_size, self.hidden_size, self.scale = int(vocab_size), int(hidden_size), float(scale)
         self.tensor_name = f"{prefix}.{weight_name}" if weight_name else prefix
         self.weight: Optional[torch.Tensor] = None
 
@@ -30,7 +32,7 @@ class TokenEmbedding(Embedding):
 
     def forward(self, tokens: torch.Tensor, ctx=None) -> torch.Tensor:
         out = ops.scratch("residual", (tokens.numel(), self.hidden_size), torch.float32, tokens.device)
-        return ops.embedding(tokens, self.weight, out)
+        return ops.embedding(tokens, self.weight, out, self.scale)
 
 
 class PairEmbedding(Embedding):
