@@ -161,6 +161,29 @@ def test_configurations_drawn_at_random(seed, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layer_sizes_of_a_larger_model(dtype, tmp_path):
+    """Two layers with heads and latents of the sizes a model of some billions of weights has (sixteen heads of
+    128 + 64 query/key dims, latents of 512 and 384, windows that a prompt of 300 tokens passes): a whole prompt (the
+    kernels for many rows), the same in portions, and a tail decoded token by token beside a second request."""
+    from gesutar_util import layer, mixer, model, moe
+    big = model(256, 1031, [
+        layer(mixer(16, 128, 64, 128, 512, 200, 64, 10000.0, 192 ** -0.5), moe(16, 4, 64, (4, 2), 1.0, 128)),
+        layer(mixer(32, 64, 32, 64, 384, 90, 32, 500000.0, 96 ** -0.5), moe(12, 3, 32, (3, 2), 2.0, None)),
+    ], bigram=(4093, 31, 17), scale=8.0)
+    cfg = every_expert(big) if dtype == "bfloat16" else big
+    folder, w = make_folder(tmp_path, cfg, seed=5, store=torch.bfloat16 if dtype == "bfloat16" else torch.float32,
+                            sharpen=1.0 if dtype == "bfloat16" else 3.0)
+    w64 = rounded(w) if dtype == "bfloat16" else as_double(w)
+    reqs = {"long": random_tokens(300, cfg["vocab"], 1), "short": random_tokens(45, cfg["vocab"], 2)}
+    ref = {rid: plain.forward(cfg, w64, toks) for rid, toks in reqs.items()}
+    runner = make_runner(folder, dtype, 16, 384 + 64)
+    for st in (traces.whole(reqs), traces.portions(reqs), traces.mixed(reqs, seed=1)[0]):
+        worst = check(replay(runner, st), st, ref, TOL[dtype])
+        assert all_free(runner)
+        print(f"larger sizes {dtype}: worst {worst:.2e}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_captured_steps(dtype, tmp_path_factory):
     """The same cuttings with every step as a HIP graph of its shape (padding tokens, requests and
     rows), twice over so that the second pass replays what the first captured."""
