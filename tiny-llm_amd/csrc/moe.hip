@@ -1,6 +1,8 @@
-// A mixture of small gated feed-forward layers whose experts are looked up in a table by token id (no
-// router): every token uses `top` experts with equal weights.  The products here are rows against the
-// weights of each row's own expert; the activation between them is the gated unit's kernel.
+// Mixtures of small feed-forward layers.  The experts of a token are named by a table: looked up by token id (no
+// router, equal weights), or a row per token of the step that a router has just filled (`moe_route_kernel`: softmax
+// scores, groups of experts, the best of the best groups, weights from the scores).  The products here are rows
+// against the weights of each row's own expert, for few rows one row at a time, for many rows sorted by expert;
+// the activation between them is a kernel of its own or rides in the first product.
 //
 // A row's sums are formed in one fixed order (the lanes of a wave stride over the inner size, then a
 // butterfly), whatever else the step holds.  Accumulation is float32 in both precisions.
@@ -10,7 +12,10 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / TL_WAVE;
-constexpr int kCols = 64;                 // output columns a workgroup owns, kCols / kWaves a wave
+// Output columns a workgroup of the per-row products owns (a quarter of them a wave): 64, or 16 in steps of few
+// rows, whose waves then form one group of four sums each instead of four in a row (the grid is four times larger,
+// and a decode step's handful of rows still fills the chip).
+constexpr int kColsWide = 64, kColsFew = 16, kFewRows = 256;
 
 __device__ __forceinline__ float dot_lanes(const float* __restrict__ a, const float* __restrict__ w, int K, int lane) {
   float acc = 0.f;
@@ -125,7 +130,8 @@ __global__ __launch_bounds__(kThreads) void table_moe_up_kernel(const T* __restr
                                                                 const T* __restrict__ w,
                                                                 const int32_t* __restrict__ tokens,
                                                                 const int32_t* __restrict__ table, T* __restrict__ out,
-                                                                int top, int experts, int vocab, int N, int K, int act) {
+                                                                int top, int experts, int vocab, int N, int K, int act,
+                                                                int kCols) {
   const int row = blockIdx.x, t = row / top, j = row - t * top;
   const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
   const int e = expert_of(tokens, table, t, j, top, vocab, experts);
@@ -152,7 +158,7 @@ __global__ __launch_bounds__(kThreads) void table_moe_down_kernel(const T* __res
                                                                   const float* __restrict__ base_scale,
                                                                   const float* __restrict__ row_w,
                                                                   float* __restrict__ out, int top, int experts,
-                                                                  int vocab, int N, int K, float coef) {
+                                                                  int vocab, int N, int K, float coef, int kCols) {
   const int t = blockIdx.x;
   const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
   const int n0 = blockIdx.y * kCols + wave * (kCols / kWaves);
@@ -578,15 +584,16 @@ int tl_table_moe_up(const void* a, int64_t a_stride, const void* w, const int32_
   if (n_tokens <= 0) return TL_OK;
   if (top <= 0 || experts <= 0 || vocab <= 0 || N <= 0 || K <= 0 || a_stride < K || !a || !w || !table || !out ||
       (act != kActNone && act != kActRelu2) || (!tokens && vocab < n_tokens) ||
-      (int64_t)n_tokens * top > 0x7fffffff || (N + kCols - 1) / kCols > 65535)
+      (int64_t)n_tokens * top > 0x7fffffff || (N + kColsFew - 1) / kColsFew > 65535)
     return TL_ERR_ARG;
+  const int kCols = (int64_t)n_tokens * top <= kFewRows ? kColsFew : kColsWide;
   dim3 g(n_tokens * top, (N + kCols - 1) / kCols), b(kThreads);
   if (dtype == 0)
     hipLaunchKernelGGL(table_moe_up_kernel<float>, g, b, 0, stream, (const float*)a, a_stride, (const float*)w, tokens,
-                       table, (float*)out, top, experts, vocab, N, K, act);
+                       table, (float*)out, top, experts, vocab, N, K, act, kCols);
   else if (dtype == 1)
     hipLaunchKernelGGL(table_moe_up_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)a, a_stride, (const bf16_t*)w, tokens,
-                       table, (bf16_t*)out, top, experts, vocab, N, K, act);
+                       table, (bf16_t*)out, top, experts, vocab, N, K, act, kCols);
   else
     return TL_ERR_ARG;
   return tl_launch_status();
@@ -600,15 +607,16 @@ int tl_table_moe_down(const void* z, const void* w, const int32_t* tokens, const
   if (n_tokens <= 0) return TL_OK;
   if (top <= 0 || experts <= 0 || vocab <= 0 || N <= 0 || K <= 0 || !z || !w || !table || !out ||
       (!tokens && vocab < n_tokens) ||
-      (N + kCols - 1) / kCols > 65535)
+      (N + kColsFew - 1) / kColsFew > 65535)
     return TL_ERR_ARG;
+  const int kCols = (int64_t)n_tokens * top <= kFewRows ? kColsFew : kColsWide;
   dim3 g(n_tokens, (N + kCols - 1) / kCols), b(kThreads);
   if (dtype == 0)
     hipLaunchKernelGGL(table_moe_down_kernel<float>, g, b, 0, stream, (const float*)z, (const float*)w, tokens, table,
-                       base, base_scale, row_w, out, top, experts, vocab, N, K, coef);
+                       base, base_scale, row_w, out, top, experts, vocab, N, K, coef, kCols);
   else if (dtype == 1)
     hipLaunchKernelGGL(table_moe_down_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)z, (const bf16_t*)w, tokens, table,
-                       base, base_scale, row_w, out, top, experts, vocab, N, K, coef);
+                       base, base_scale, row_w, out, top, experts, vocab, N, K, coef, kCols);
   else
     return TL_ERR_ARG;
   return tl_launch_status();
