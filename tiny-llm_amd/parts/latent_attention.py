@@ -139,6 +139,10 @@ class LatentAttention(Mixer):
         # the same two as [heads, inner, cols], for the one-launch products of steps with few rows
         self.w_uk_few = ops.head_product_weights(uk)
         self.w_uv_few = ops.head_product_weights(self.w_uv.view(H, self.value_dim, self.kv_rank).transpose(1, 2))
+        # for steps of few rows the value products are rows against the weights of each row's own head: row t * H + n
+        # takes head n (the table the per-row kernel of the experts looks its weights up in)
+        self.head_of_row = (torch.arange(ops.HEAD_PRODUCT_ROWS * H, dtype=torch.int32, device=self.w_uv.device) % H
+                            ).reshape(-1, 1).contiguous()
         self.w_o = tensors[n["o"]].contiguous()
 
     def cache_spec(self) -> CacheSpec:
@@ -222,7 +226,13 @@ class LatentAttention(Mixer):
         V, dev = self.value_dim, mix.device
         o = ops.scratch("latent_heads", (T, H * V), self.dtype, dev)
         gate = down[:, self.g_off:self.g_off + H * V] if self.gate == "element" else None
-        if few:
+        if few and KR >= 256:
+            # a long inner size and few columns a head: a wave a group of four columns of one (token, head), its lanes
+            # striding over the latent, fills the chip where a workgroup per 64 columns of a head leaves it idle
+            ops.table_moe_up(mix.view(T * H, KR), self.w_uv.view(H, V, KR), None, self.head_of_row, o.view(T * H, V))
+            if gate is not None:
+                ops.gate_rows(o, gate, o)
+        elif few:
             ops.head_products(mix, self.w_uv_few, o.view(T, H, V), gate)      # the gate rides in the product
         elif many:
             ops.head_gemm(mix, self.w_uv.view(H, V, KR), o.view(T, H, V), gate)
