@@ -104,6 +104,31 @@ def test_refusals():
         _decoder(cfg, "bfloat16")
 
 
+def test_sizes_the_bfloat16_kernels_refuse_are_served_in_float32():
+    """The front ends' builder: a bfloat16 engine given a model with rows of no multiple of 8 elements builds
+    the float32 decoder and warns, naming the size; sizes that both refuse are refused; a model that fits is
+    built as asked."""
+    from tiny_llm_amd.engine.loading import build_decoder
+    from tiny_llm_amd.kernels.ops import KernelError
+    with pytest.warns(RuntimeWarning, match="served in float32.*hidden_size = 50"):
+        _, dec = build_decoder(ODD, "bfloat16", "cpu")
+    assert dec.dtype == torch.float32
+    cfg = copy.deepcopy(MIX_A)
+    cfg["layers"][0]["mlp"]["expert"]["ff"] = 20
+    with pytest.warns(RuntimeWarning, match="intermediate_size = 20"):
+        assert build_decoder(cfg, "bfloat16", "cpu")[1].dtype == torch.float32
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        assert build_decoder(MIX_A, "bfloat16", "cpu")[1].dtype == torch.bfloat16
+        assert build_decoder(ODD, "float32", "cpu")[1].dtype == torch.float32
+    cfg = copy.deepcopy(MIX_A)
+    cfg["layers"][0]["mixer"]["kv_rank"] = 100000
+    for dtype in ("bfloat16", "float32"):
+        with pytest.raises(KernelError):
+            build_decoder(cfg, dtype, "cpu")
+
+
 def test_configurations_drawn_at_random_build():
     for seed in range(30):
         cfg = random_config(seed)

@@ -121,6 +121,22 @@ def test_whole_tail_portions(name, dtype, tmp_path_factory):
         assert all_free(runner)
 
 
+def test_odd_sizes_in_a_bfloat16_engine(tmp_path_factory):
+    """A checkpoint stored in bfloat16 whose sizes are multiples of nothing, asked for in bfloat16: the float32
+    kernels serve it (with a warning), mixed batches and portions agree with the plain model to float32's limit."""
+    cfg, block = CONFIGS["odd"]
+    folder, w = make_folder(tmp_path_factory.mktemp("gesutar_odd_bf16"), cfg, seed=4, store=torch.bfloat16)
+    reqs = {f"r{i}": random_tokens(n, cfg["vocab"], 50 + i) for i, n in enumerate(LENGTHS["odd"])}
+    ref = {rid: plain.forward(cfg, rounded(w), toks) for rid, toks in reqs.items()}
+    steps, peak = traces.mixed(reqs, seed=3)
+    with pytest.warns(RuntimeWarning, match="served in float32"):
+        runner = make_runner(folder, "bfloat16", block, max(peak, max(r64(len(t)) for t in reqs.values())))
+    assert runner.decoder.dtype == torch.float32
+    for st in (steps, traces.portions(reqs)):
+        check(replay(runner, st), st, ref, TOL["float32"])
+        assert all_free(runner)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_mixed_batches_reuse_pages_and_slots(name, dtype, tmp_path_factory):

@@ -2,6 +2,7 @@
 and a runner: the one way every front end (generation, replay, bench) builds a model."""
 from __future__ import annotations
 
+import warnings
 from typing import Mapping, Optional, Sequence
 
 import torch
@@ -9,6 +10,7 @@ import torch
 from ..cache import CacheManager
 from ..config import EngineConfig, resolve, read_config_json
 from ..kernels import library
+from ..kernels.ops import KernelError
 from ..models.decoder import Decoder
 from ..weights import Checkpoint, init_random_weights, load_weights
 from .step import ModelRunner
@@ -27,8 +29,21 @@ def require_gpu(device: int = 0) -> torch.device:
 
 
 def build_decoder(config: Mapping, dtype: str, device, tensor_shapes: Optional[Mapping] = None) -> tuple:
+    """A model whose sizes the bfloat16 kernels refuse (they move 16-byte vectors: rows of a multiple of 8
+    elements) is served by the float32 kernels, which take any size, and a warning says so; a model that
+    those refuse as well is refused."""
     cfg, spec = resolve(config, tensor_shapes)
-    return cfg, Decoder(spec, dtype=dtype, device=device)
+    try:
+        return cfg, Decoder(spec, dtype=dtype, device=device)
+    except KernelError as refusal:
+        if dtype not in ("bfloat16", torch.bfloat16):
+            raise
+        try:
+            dec = Decoder(spec, dtype="float32", device=device)
+        except KernelError:
+            raise refusal from None
+        warnings.warn(f"{spec.architecture}: served in float32, since {refusal}", RuntimeWarning, stacklevel=2)
+        return cfg, dec
 
 
 def load_model(model_path: str, engine: EngineConfig):
