@@ -2,6 +2,7 @@ from .llama import LlamaConfig, ConfigError
 from .lufazen import LufazenConfig
 from .fofapel import FofapelConfig
 from .gesutar import GesutarConfig
+from .vevapel import VevapelConfig
 from .engine import EngineConfig
 from .spec import PartSpec, LayerSpec, PlanEntry, ModelSpec, pre_norm_layer
 from .registry import (register_architecture, unregister_architecture, known_architectures,

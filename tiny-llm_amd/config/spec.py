@@ -52,9 +52,12 @@ def pre_norm_layer(prefix: str, mixer_norm: PartSpec, mixer: PartSpec, ffn_norm:
 @dataclass(frozen=True)
 class PlanEntry:
     """One run of a layer.  `cache_of` names an earlier plan entry whose cache
-    this run reads instead of keeping its own (it then writes nothing)."""
+    this run reads instead of keeping its own (it then writes nothing).  `before` = (i, turn): ahead of
+    this run the residual stream passes through `ModelSpec.stream_parts[i]`, which is told `turn`
+    (the number of the pass through a run of layers that the model repeats, for instance)."""
     layer: int
     cache_of: Optional[int] = None
+    before: Optional[Tuple[int, int]] = None
 
 
 @dataclass(frozen=True)
@@ -71,6 +74,9 @@ class ModelSpec:
     eos_token_ids: Tuple[int, ...] = ()
     # glob patterns of tensors that checkpoints of this architecture carry and no part needs
     ignorable_tensors: Tuple[str, ...] = ()
+    # parts that act on the residual stream between layer runs (plan entries name them in `before`);
+    # a part's `name` is its whole weight prefix
+    stream_parts: Tuple[PartSpec, ...] = ()
 
     def validate(self) -> None:
         n = len(self.layers)
@@ -82,6 +88,9 @@ class ModelSpec:
         for i, e in enumerate(self.plan):
             if not (0 <= e.layer < n):
                 raise ValueError(f"plan entry {i} names layer {e.layer}, model has {n}")
+            if e.before is not None:
+                if not (0 <= e.before[0] < len(self.stream_parts)):
+                    raise ValueError(f"plan entry {i} names stream part {e.before[0]}, model has {len(self.stream_parts)}")
             if e.cache_of is not None:
                 if not (0 <= e.cache_of < i):
                     raise ValueError(

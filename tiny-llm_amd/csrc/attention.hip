@@ -21,6 +21,15 @@
 
 namespace {
 
+// The first key position a row at position `pos` sees (it sees up to its own): with window > 0 the last
+// `window` positions; with window < 0 its own run of -window positions, runs counted from position 0 of
+// the sequence (a chunked mask); with 0 everything.  Never decreases as pos grows.
+__device__ __forceinline__ int first_visible_key(int pos, int window) {
+  if (window > 0) return pos + 1 > window ? pos + 1 - window : 0;
+  if (window < 0 && pos > 0) return pos / (-window) * (-window);
+  return 0;
+}
+
 constexpr int kMaxHd = 256;
 constexpr int kDPL = kMaxHd / TL_WAVE;  // output dims per lane
 
@@ -36,7 +45,7 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
   const int r = req_of_token[t];
   const int pos = positions[t];
   const int kv_end = pos + 1;
-  const int kv_begin = (window > 0 && kv_end > window) ? kv_end - window : 0;
+  const int kv_begin = first_visible_key(pos, window);
   const int kvh = h / (nq / nkv);
   const int32_t* bt = block_tables + (int64_t)r * max_blocks;
 
@@ -239,7 +248,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
       if (do_rope) qy[ks] = *(const bf16x8*)(qrow + dp);      // uniform
     }
   }
-  const int row_lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int row_lo = first_visible_key(pos, window);
 
   // key range of the tile: union over its rows
   const int hi = row_max_i32(pos), lo = row_min_i32(row_valid ? row_lo : 0x7fffffff);
@@ -732,7 +741,7 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
   const bool row_valid = tok_local < TW && tok_local < ntok;
   const int tok = tok0 + (row_valid ? tok_local : 0);
   const int pos = row_valid ? positions[tok] : -1;
-  const int row_lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int row_lo = first_visible_key(pos, window);
   const int hi = row_max_i32(pos), lo = row_min_i32(row_valid ? row_lo : 0x7fffffff);
   const int kv_end = hi + 1, kv_begin = lo;
   const int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
@@ -842,7 +851,7 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_rows_kernel(
   const bool row_valid = tok_local < TW && tok_local < ntok;
   const int tok = tok0 + (row_valid ? tok_local : 0);
   const int pos = row_valid ? positions[tok] : -1;
-  const int row_lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int row_lo = first_visible_key(pos, window);
   const int hi = row_max_i32(pos), lo = row_min_i32(row_valid ? row_lo : 0x7fffffff);
   const int kv_end = hi + 1, kv_begin = lo;
   const int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
@@ -960,7 +969,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
   // the tokens of a tile are consecutive tokens of one request, so their positions are consecutive
   const int pos_first = positions[tok0], pos_last = pos_first + ntok - 1;
   const int kv_end = pos_last + 1;
-  const int kv_begin = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
+  const int kv_begin = first_visible_key(pos_first, window);
   int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
   if (n_splits > 1) {       // this workgroup's share of the key tiles (possibly none)
     const int per = (last_tile - first_tile + n_splits - 1) / n_splits;
@@ -979,7 +988,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
     row_valid[rt] = r16 / G < TW && tok_local < ntok;
     tok[rt] = tok0 + (row_valid[rt] ? tok_local : 0);
     pos[rt] = row_valid[rt] ? pos_first + tok_local : -1;
-    row_lo[rt] = (window > 0 && pos[rt] + 1 > window) ? pos[rt] + 1 - window : 0;
+    row_lo[rt] = first_visible_key(pos[rt], window);
     const bf16_t* qrow = q + (int64_t)tok[rt] * q_stride + (int64_t)head * HD;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -1399,7 +1408,7 @@ int tl_paged_attention(const void* q, int64_t q_stride, const void* k_cache, con
                        hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (nq <= 0 || nkv <= 0 || nq % nkv || hd <= 0 || hd > kMaxHd || block_size <= 0 || max_blocks <= 0 ||
-      window < 0 || nq > 65535)
+      nq > 65535)
     return TL_ERR_ARG;
   dim3 g(n_tokens, nq), b(TL_WAVE);
   if (dtype == 0)
@@ -1426,7 +1435,7 @@ int tl_attention_f32(const float* q, int64_t q_stride, const float* k_cache, con
                      int block_size, float scale, int window, int sink, int n_chunks, hipStream_t stream) {
   if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
   if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
-      max_blocks <= 0 || window < 0 || n_chunks < 1 || nkv > 65535 || n_chunks > 65535 || q_stride % 4 ||
+      max_blocks <= 0 || n_chunks < 1 || nkv > 65535 || n_chunks > 65535 || q_stride % 4 ||
       out_stride % 1)
     return TL_ERR_ARG;
   if (n_chunks > 1 && !part) return TL_ERR_ARG;
@@ -1499,7 +1508,7 @@ int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const
       (int64_t)n_tiles * nkv * n_splits > 0x7fffffff)
     return TL_ERR_ARG;
   if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
-      max_blocks <= 0 || window < 0 || nkv > 65535 || (int64_t)n_tiles * nkv > 0x7fffffff || q_stride % 8 ||
+      max_blocks <= 0 || nkv > 65535 || (int64_t)n_tiles * nkv > 0x7fffffff || q_stride % 8 ||
       out_stride % 4)
     return TL_ERR_ARG;
   int bs_shift = -1;      // log2 of the page size where it is a power of two
@@ -1548,7 +1557,7 @@ static int flash_attention_any(const void* q, int64_t q_stride, const void* k_ca
                                const float* rope_cos, const float* rope_sin, int fuse_store, hipStream_t stream) {
   if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
   if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
-      max_blocks <= 0 || window < 0 || n_splits < 1 || nkv > 65535 || n_splits > 65535 || q_stride % 8)
+      max_blocks <= 0 || n_splits < 1 || nkv > 65535 || n_splits > 65535 || q_stride % 8)
     return TL_ERR_ARG;
   if (n_splits > 1 && (!part_o || !part_ml)) return TL_ERR_ARG;
   if (!tile_req && (tile_tok0 || tile_ntok || n_tiles != n_tokens)) return TL_ERR_ARG;

@@ -1,4 +1,5 @@
-// The gated delta rule with one decay per head and key channel, as a recurrence over a state
+// The gated delta rule with one decay per head and key channel (or one per head, laid out over the
+// channels where the recurrence reads it), as a recurrence over a state
 // S [dim, vdim] per request and head:
 //     S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
 // and what surrounds it: short causal convolutions with SiLU on q, k and v (their last taps - 1
@@ -50,7 +51,8 @@ __device__ __forceinline__ float conv_silu(const T* __restrict__ p, int64_t p_st
 
 // One workgroup per (token, head).  Row t of `p` holds [q (kv_heads x dim) | k (kv_heads x dim) |
 // v (heads x vdim)] from column conv_off on, and beta's pre-activation at column b_off + head;
-// row t of `a` holds the decay's pre-activation at column head * dim + i.
+// row t of `a` holds the decay's pre-activation at column head * dim + i, or, with a_per_head, one per
+// head at column head (dt_bias is indexed likewise).
 template <typename T>
 __global__ __launch_bounds__(kPrepThreads) void delta_prepare_kernel(
     const T* __restrict__ p, int64_t p_stride, int conv_off, int b_off, const float* __restrict__ a, int64_t a_stride,
@@ -58,7 +60,7 @@ __global__ __launch_bounds__(kPrepThreads) void delta_prepare_kernel(
     const float* __restrict__ state, int64_t state_stride, int64_t saved_off, const int32_t* __restrict__ req_of_token,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, float* __restrict__ qn,
     float* __restrict__ kn, float* __restrict__ vc, float* __restrict__ beta, float* __restrict__ decay, int heads,
-    int kv_heads, int dim, int vdim, int taps, float q_scale) {
+    int kv_heads, int dim, int vdim, int taps, float q_scale, int a_per_head) {
   __shared__ float qs[kMaxDim], ks[kMaxDim], red[kPrepWaves];
   const int t = blockIdx.x, h = blockIdx.y;
   const int r = req_of_token[t];
@@ -92,7 +94,8 @@ __global__ __launch_bounds__(kPrepThreads) void delta_prepare_kernel(
   for (int i = threadIdx.x; i < dim; i += kPrepThreads) {
     qn[base * dim + i] = qs[i] * rq;
     kn[base * dim + i] = ks[i] * rk;
-    const float pre = a[(int64_t)t * a_stride + h * dim + i] + dt_bias[h * dim + i];
+    const int ai = a_per_head ? h : h * dim + i;
+    const float pre = a[(int64_t)t * a_stride + ai] + dt_bias[ai];
     decay[base * dim + i] = expf(-rate * softplus(pre));
   }
   for (int j = threadIdx.x; j < vdim; j += kPrepThreads)
@@ -277,7 +280,7 @@ __device__ __forceinline__ float block_sum_dyn(float v, float* red, int nw) {
 // A decode step in one kernel: every request brings ONE token.  One workgroup per (request, head),
 // a thread per value column: the convolutions, unit vectors, decay and beta of the token, the
 // recurrence on the column in registers, and the head's norm and gate on the way out
-// (z[t, h, :] = w * o / rms(o) * sigmoid(gate)).  The saved convolution inputs are brought up to date
+// (z[t, h, :] = w * o / rms(o) * act(gate), act the sigmoid or, with gate_kind 1, g * sigmoid(g)).  The saved convolution inputs are brought up to date
 // here when every head has q/k channels of its own (update_saved); else several workgroups read a
 // channel's saved inputs and conv_state_update_kernel runs behind this kernel.
 constexpr int kDecodeThreads = 256;     // value columns the one-kernel decode step takes (a thread each)
@@ -309,12 +312,13 @@ __device__ __forceinline__ void store_saved(float* __restrict__ saved, const flo
 // State phase of the kernel: thread (sl, cq) keeps rows [sl * DS, (sl + 1) * DS) of the FOUR value columns
 // 4 cq .. 4 cq + 3 of S in registers (16-byte loads and stores: a lane that moves four bytes at a time gets a
 // fraction of what a compute unit can fetch), the four slices' partial sums meet in LDS in a fixed order.
-template <typename T, int DS>
+template <typename T, typename TZ, int DS>
 __global__ __launch_bounds__(kDecodeThreads) void delta_decode_kernel(
-    const T* __restrict__ p, int64_t p_stride, int conv_off, int b_off, const float* __restrict__ low, int64_t low_stride,
+    const T* __restrict__ p, int64_t p_stride, int conv_off, int b_off, const float* __restrict__ a, int64_t a_stride,
+    int a_per_head, const float* __restrict__ gate, int64_t gate_stride, int gate_kind,
     const float* __restrict__ conv_w, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
     const float* __restrict__ w_norm, float* __restrict__ state, int64_t state_stride, int64_t saved_off,
-    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, T* __restrict__ z, int heads,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, TZ* __restrict__ z, int heads,
     int kv_heads, int dim, int vdim, int taps, float q_scale, float eps, int update_saved) {
   __shared__ float qs[kMaxDim], ks[kMaxDim], gs[kMaxDim], vs[kDecodeThreads], red[16];
   __shared__ f32x4 part[4][kDecodeThreads / 4];
@@ -338,13 +342,14 @@ __global__ __launch_bounds__(kDecodeThreads) void delta_decode_kernel(
   load_taps(p, p_stride, t, conv_off + q_ch + i0, sv_q, conv_w + (int64_t)(q_ch + i0) * taps, taps, xq, wq);
   load_taps(p, p_stride, t, conv_off + k_ch + i0, sv_k, conv_w + (int64_t)(k_ch + i0) * taps, taps, xk, wk);
   load_taps(p, p_stride, t, conv_off + v_ch + c0, sv_v, conv_w + (int64_t)(v_ch + c0) * taps, taps, xv, wv);
-  const float pre_a = low[(int64_t)t * low_stride + h * dim + i0] + dt_bias[h * dim + i0];
+  const int ai = a_per_head ? h : h * dim + i0;
+  const float pre_a = a[(int64_t)t * a_stride + ai] + dt_bias[ai];
   const float pre_b = to_f32(p[(int64_t)t * p_stride + b_off + h]);
   const float rate = expf(a_log[h]);
   float pre_g[4], wn[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    pre_g[e] = low[(int64_t)t * low_stride + heads * dim + h * vdim + cq * 4 + e];
+    pre_g[e] = gate[(int64_t)t * gate_stride + h * vdim + cq * 4 + e];
     wn[e] = w_norm[cq * 4 + e];
   }
   float* S_mem = row + (int64_t)h * dim * vdim + cq * 4;
@@ -429,8 +434,10 @@ __global__ __launch_bounds__(kDecodeThreads) void delta_decode_kernel(
   if (sl == 0) {
     const float rn = 1.f / sqrtf(ss / (float)vdim + eps);
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-      z[((int64_t)t * heads + h) * vdim + cq * 4 + e] = from_f32<T>(o[e] * rn * wn[e] / (1.f + expf(-pre_g[e])));
+    for (int e = 0; e < 4; ++e) {
+      const float sg = 1.f / (1.f + expf(-pre_g[e]));
+      z[((int64_t)t * heads + h) * vdim + cq * 4 + e] = from_f32<TZ>(o[e] * rn * wn[e] * (gate_kind ? pre_g[e] * sg : sg));
+    }
   }
 }
 
@@ -447,8 +454,8 @@ int tl_delta_prepare(const void* p, int64_t p_stride, int conv_off, int b_off, c
                      const float* conv_w, const float* a_log, const float* dt_bias, const float* state,
                      int64_t state_stride, int64_t saved_off, const int32_t* req_of_token, const int32_t* cu_seqlens,
                      const int32_t* state_slots, float* qn, float* kn, float* vc, float* beta, float* decay,
-                     int n_tokens, int heads, int kv_heads, int dim, int vdim, int taps, float q_scale, int dtype,
-                     hipStream_t stream) {
+                     int n_tokens, int heads, int kv_heads, int dim, int vdim, int taps, float q_scale, int a_per_head,
+                     int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (heads <= 0 || heads > 65535 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || dim > kMaxDim || vdim <= 0 ||
       taps < 1 || taps > kMaxTaps)
@@ -457,7 +464,7 @@ int tl_delta_prepare(const void* p, int64_t p_stride, int conv_off, int b_off, c
   TL_DISPATCH_T(dtype, hipLaunchKernelGGL(delta_prepare_kernel<T>, g, b, 0, stream, (const T*)p, p_stride, conv_off,
                                           b_off, a, a_stride, conv_w, a_log, dt_bias, state, state_stride, saved_off,
                                           req_of_token, cu_seqlens, state_slots, qn, kn, vc, beta, decay, heads,
-                                          kv_heads, dim, vdim, taps, q_scale);)
+                                          kv_heads, dim, vdim, taps, q_scale, a_per_head);)
   return tl_launch_status();
 }
 
@@ -492,31 +499,35 @@ int tl_delta_recurrence(const float* qn, const float* kn, const float* vc, const
   return tl_launch_status();
 }
 
-// `low` row t: [decay pre-activations heads x dim | gate pre-activations heads x vdim], float32.
-int tl_delta_decode(const void* p, int64_t p_stride, int conv_off, int b_off, const float* low, int64_t low_stride,
-                    const float* conv_w, const float* a_log, const float* dt_bias, const float* w_norm, float* state,
+// Row t of `a`: the decay's pre-activations (heads x dim, or heads with a_per_head); of `gate`: the gate's (heads x
+// vdim); both float32.
+int tl_delta_decode(const void* p, int64_t p_stride, int conv_off, int b_off, const float* a, int64_t a_stride,
+                    int a_per_head, const float* gate, int64_t gate_stride, int gate_kind, const float* conv_w, const float* a_log, const float* dt_bias, const float* w_norm, float* state,
                     int64_t state_stride, int64_t saved_off, const int32_t* cu_seqlens, const int32_t* state_slots,
                     void* z, int n_requests, int heads, int kv_heads, int dim, int vdim, int taps, float q_scale,
-                    float eps, int update_saved, int dtype, hipStream_t stream) {
+                    float eps, int update_saved, int dtype, int z_dtype, hipStream_t stream) {
   if (n_requests <= 0) return TL_OK;
   if (heads <= 0 || heads > 65535 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || dim > kMaxDim || vdim <= 0 ||
       vdim > kDecodeThreads || vdim % 4 || state_stride % 4 || dim > kDecodeThreads || taps < 1 || taps > 4 ||
-      (update_saved && heads != kv_heads))
+      (update_saved && heads != kv_heads) || gate_kind < 0 || gate_kind > 1 || !a || !gate)
     return TL_ERR_ARG;
   const int threads = vdim > dim ? vdim : dim;      // a thread per value column and per key channel
   dim3 g(n_requests, heads), b((threads + TL_WAVE - 1) / TL_WAVE * TL_WAVE);
-#define TL_DEC(TT, D)                                                                                               \
-  hipLaunchKernelGGL((delta_decode_kernel<TT, D>), g, b, 0, stream, (const TT*)p, p_stride, conv_off, b_off, low,   \
-                     low_stride, conv_w, a_log, dt_bias, w_norm, state, state_stride, saved_off, cu_seqlens,        \
-                     state_slots, (TT*)z, heads, kv_heads, dim, vdim, taps, q_scale, eps, update_saved)
-#define TL_DEC_D(TT)                  \
-  if (dim <= 16) TL_DEC(TT, 4);       \
-  else if (dim <= 32) TL_DEC(TT, 8);  \
-  else if (dim <= 64) TL_DEC(TT, 16); \
-  else if (dim <= 128) TL_DEC(TT, 32); \
-  else TL_DEC(TT, 64);
-  if (dtype == 0) { TL_DEC_D(float) }
-  else if (dtype == 1) { TL_DEC_D(bf16_t) }
+#define TL_DEC(TT, TZ, D)                                                                                          \
+  hipLaunchKernelGGL((delta_decode_kernel<TT, TZ, D>), g, b, 0, stream, (const TT*)p, p_stride, conv_off, b_off, a, \
+                     a_stride, a_per_head, gate, gate_stride, gate_kind, conv_w, a_log, dt_bias, w_norm, state,     \
+                     state_stride, saved_off, cu_seqlens, state_slots, (TZ*)z, heads, kv_heads, dim, vdim, taps,    \
+                     q_scale, eps, update_saved)
+#define TL_DEC_D(TT, TZ)                  \
+  if (dim <= 16) TL_DEC(TT, TZ, 4);       \
+  else if (dim <= 32) TL_DEC(TT, TZ, 8);  \
+  else if (dim <= 64) TL_DEC(TT, TZ, 16); \
+  else if (dim <= 128) TL_DEC(TT, TZ, 32); \
+  else TL_DEC(TT, TZ, 64);
+  // the projections' element type and the result's: float32 projections may feed a bfloat16 output product
+  if (dtype == 0 && z_dtype == 0) { TL_DEC_D(float, float) }
+  else if (dtype == 0 && z_dtype == 1) { TL_DEC_D(float, bf16_t) }
+  else if (dtype == 1 && z_dtype == 1) { TL_DEC_D(bf16_t, bf16_t) }
   else return TL_ERR_ARG;
 #undef TL_DEC_D
 #undef TL_DEC

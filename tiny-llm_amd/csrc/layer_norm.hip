@@ -1,7 +1,9 @@
 // Layer norm with weight and bias, (v - mean) / sqrt(var + eps) * w + b with var the mean squared
 // deviation, in two forms: on the sum of a sublayer's result and the scaled residual stream, written
 // back into the stream (a layer whose norm FOLLOWS the sum: x <- LN(alpha * x + y)), and on gathered
-// rows of the stream for the output head.
+// rows of the stream for the output head; and on a sublayer's result by itself, added to the stream times a
+// constant (a layer with a norm in front of AND behind every sublayer: x <- x + m * LN(y)), with the norm that
+// reads the new stream next in the same pass over the row.
 //
 // Statistics, weight, bias and the stream are float32 in both precisions.  The mean is taken first and
 // the variance from the deviations (two sums), not from the mean of squares.
@@ -72,6 +74,78 @@ __global__ __launch_bounds__(kThreads) void layer_norm_kernel(const float* __res
   }
 }
 
+// x[row] <- x[row] + mult * (LN(y[row]) * w + b); then, if w2 is given, out[row] = LN(x[row]) * w2 + b2 in TO: the
+// norm of whatever reads the stream next, formed while the row is in registers.  One workgroup a row; rows of up
+// to KEEP * kThreads elements.
+template <typename TO, int KEEP>
+__global__ __launch_bounds__(kThreads) void layer_norm_add_kernel(const float* __restrict__ y, const float* __restrict__ w,
+                                                                  const float* __restrict__ b, float* __restrict__ x,
+                                                                  const float* __restrict__ w2, const float* __restrict__ b2,
+                                                                  TO* __restrict__ out, int hidden, float mult, float eps,
+                                                                  float eps2) {
+  __shared__ float red[kWaves];
+  const int64_t row = blockIdx.x;
+  float* xr = x + row * hidden;
+  const float* yr = y + row * hidden;
+  const float inv_n = 1.f / (float)hidden;
+  float v[KEEP];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int j = threadIdx.x + i * kThreads;
+    v[i] = j < hidden ? yr[j] : 0.f;
+    s += v[i];
+  }
+  float mean = block_sum<kWaves>(s, red) * inv_n;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int j = threadIdx.x + i * kThreads;
+    const float d = j < hidden ? v[i] - mean : 0.f;
+    q += d * d;
+  }
+  float r = 1.f / sqrtf(block_sum<kWaves>(q, red) * inv_n + eps);
+  s = 0.f;
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int j = threadIdx.x + i * kThreads;
+    if (j < hidden) {
+      v[i] = fmaf(mult, (v[i] - mean) * r * w[j] + b[j], xr[j]);
+      xr[j] = v[i];
+    } else {
+      v[i] = 0.f;
+    }
+    s += v[i];
+  }
+  if (!w2) return;
+  mean = block_sum<kWaves>(s, red) * inv_n;
+  q = 0.f;
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int j = threadIdx.x + i * kThreads;
+    const float d = j < hidden ? v[i] - mean : 0.f;
+    q += d * d;
+  }
+  r = 1.f / sqrtf(block_sum<kWaves>(q, red) * inv_n + eps2);
+  TO* dst = out + row * hidden;
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int j = threadIdx.x + i * kThreads;
+    if (j < hidden) dst[j] = from_f32<TO>((v[i] - mean) * r * w2[j] + b2[j]);
+  }
+}
+
+template <typename TO>
+int launch_add(const float* y, const float* w, const float* b, float* x, const float* w2, const float* b2, TO* out, int n,
+               int hidden, float mult, float eps, float eps2, hipStream_t stream) {
+  dim3 g(n), blk(kThreads);
+  if (hidden <= 8 * kThreads)
+    hipLaunchKernelGGL((layer_norm_add_kernel<TO, 8>), g, blk, 0, stream, y, w, b, x, w2, b2, out, hidden, mult, eps, eps2);
+  else
+    hipLaunchKernelGGL((layer_norm_add_kernel<TO, 32>), g, blk, 0, stream, y, w, b, x, w2, b2, out, hidden, mult, eps, eps2);
+  return tl_launch_status();
+}
+
 template <typename TO>
 int launch(const float* y, const float* w, const float* b, float* x, const int32_t* rows, TO* out, int n, int hidden,
            float alpha, float eps, int inplace, hipStream_t stream) {
@@ -95,6 +169,18 @@ int tl_layer_norm_sum(const float* y, const float* w, const float* b, float* x, 
   if (hidden <= 0 || !w || !b || !x) return TL_ERR_ARG;
   if (copy_dtype == 1) return launch<bf16_t>(y, w, b, x, nullptr, (bf16_t*)copy, n_rows, hidden, alpha, eps, 1, stream);
   if (copy_dtype == 0) return launch<float>(y, w, b, x, nullptr, (float*)copy, n_rows, hidden, alpha, eps, 1, stream);
+  return TL_ERR_ARG;
+}
+
+// x[t] <- x[t] + mult * (LN(y[t]) * w + b) for n_rows rows; with w2, b2 and out (out_dtype 0 float32 / 1 bfloat16)
+// also out[t] = LN(x[t]) * w2 + b2 of the new rows.  Rows of at most 8,192 elements.
+int tl_layer_norm_add(const float* y, const float* w, const float* b, float* x, const float* w2, const float* b2,
+                      void* out, int n_rows, int hidden, float mult, float eps, float eps2, int out_dtype,
+                      hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (hidden <= 0 || hidden > 32 * kThreads || !y || !w || !b || !x || (w2 && (!b2 || !out))) return TL_ERR_ARG;
+  if (out_dtype == 1) return launch_add<bf16_t>(y, w, b, x, w2, b2, (bf16_t*)out, n_rows, hidden, mult, eps, eps2, stream);
+  if (out_dtype == 0) return launch_add<float>(y, w, b, x, w2, b2, (float*)out, n_rows, hidden, mult, eps, eps2, stream);
   return TL_ERR_ARG;
 }
 

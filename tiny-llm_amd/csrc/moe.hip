@@ -414,18 +414,23 @@ __device__ __forceinline__ Best wave_best(Best x) {
 }
 
 __global__ __launch_bounds__(TL_WAVE) void moe_route_kernel(const float* __restrict__ z, int64_t z_stride,
-                                                            int32_t* __restrict__ ids, float* __restrict__ wts,
-                                                            int experts, int top, int groups, int keep, float scale) {
+                                                            const float* __restrict__ bias, int32_t* __restrict__ ids,
+                                                            float* __restrict__ wts, int experts, int top, int groups,
+                                                            int keep, float scale) {
   __shared__ float s[kMaxRouted];         // scores; -1 once an expert is chosen or its run is out
   __shared__ float gs[kMaxRouted];        // the runs' scores
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* zr = z + (int64_t)t * z_stride;
   float m = -INFINITY;
-  for (int e = lane; e < experts; e += TL_WAVE) m = fmaxf(m, zr[e]);
+  for (int e = lane; e < experts; e += TL_WAVE) {     // the logits (a bias per expert added), kept in s for the next pass
+    const float l = bias ? zr[e] + bias[e] : zr[e];
+    s[e] = l;
+    m = fmaxf(m, l);
+  }
   m = wave_max(m);
   float sum = 0.f;
   for (int e = lane; e < experts; e += TL_WAVE) {
-    const float p = expf(zr[e] - m);
+    const float p = expf(s[e] - m);
     s[e] = p;
     sum += p;
   }
@@ -638,13 +643,13 @@ int tl_row_dot_sigmoid(const void* a, int64_t a_stride, const void* w, float* ou
 }
 
 // z: float32 [n_tokens, experts] (row stride z_stride); ids: int32 [n_tokens, top]; wts: float32 [n_tokens, top].
-int tl_moe_route(const float* z, int64_t z_stride, int32_t* ids, float* wts, int n_tokens, int experts, int top,
-                 int groups, int keep, float scale, hipStream_t stream) {
+int tl_moe_route(const float* z, int64_t z_stride, const float* bias, int32_t* ids, float* wts, int n_tokens, int experts,
+                 int top, int groups, int keep, float scale, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (experts <= 0 || experts > kMaxRouted || top <= 0 || top > experts || z_stride < experts || !z || !ids || !wts ||
       groups < 0 || (groups > 1 && (experts % groups || keep <= 0 || keep > groups || top > keep * (experts / groups))))
     return TL_ERR_ARG;
-  hipLaunchKernelGGL(moe_route_kernel, dim3(n_tokens), dim3(TL_WAVE), 0, stream, z, z_stride, ids, wts, experts, top,
+  hipLaunchKernelGGL(moe_route_kernel, dim3(n_tokens), dim3(TL_WAVE), 0, stream, z, z_stride, bias, ids, wts, experts, top,
                      groups, keep, scale);
   return tl_launch_status();
 }

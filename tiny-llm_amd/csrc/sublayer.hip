@@ -104,6 +104,20 @@ __global__ void softcap_kernel(float* __restrict__ x, int64_t total, float cap) 
   if (i < total) x[i] = cap * tanhf(x[i] / cap);
 }
 
+// Two streams side by side as the operand of one product: operand[t] = [a[t] | b[t]] rounded to T, and
+// init[t] = vec (a row that the product then adds its result to, so a vector joins every row without a kernel of
+// its own).  One thread an element of the wider of the two outputs.
+template <typename T>
+__global__ void stream_join_kernel(const float* __restrict__ a, const float* __restrict__ b, const float* __restrict__ vec,
+                                   T* __restrict__ operand, float* __restrict__ init, int64_t total, int width) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / (2 * width);
+  const int c = (int)(i - t * 2 * width);
+  operand[i] = from_f32<T>(c < width ? a[t * width + c] : b[t * width + c - width]);
+  if (c < width) init[t * width + c] = vec ? vec[c] : 0.f;
+}
+
 }  // namespace
 
 extern "C" {
@@ -177,6 +191,23 @@ int tl_softcap(float* x, int64_t total, float cap, hipStream_t stream) {
   if (!(cap > 0.f)) return TL_ERR_ARG;
   hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)ceil_div64(total, kThreads)), dim3(kThreads), 0, stream, x, total,
                      cap);
+  return tl_launch_status();
+}
+
+// a, b: float32 [n_rows, width]; operand: [n_rows, 2 * width] in dtype; init: float32 [n_rows, width] (every row
+// becomes vec, or zeros without one).
+int tl_stream_join(const float* a, const float* b, const float* vec, void* operand, float* init, int n_rows, int width,
+                   int dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (width <= 0 || !a || !b || !operand || !init) return TL_ERR_ARG;
+  const int64_t total = (int64_t)n_rows * 2 * width;
+  dim3 g((unsigned)ceil_div64(total, kThreads)), blk(kThreads);
+  if (dtype == 0)
+    hipLaunchKernelGGL(stream_join_kernel<float>, g, blk, 0, stream, a, b, vec, (float*)operand, init, total, width);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(stream_join_kernel<bf16_t>, g, blk, 0, stream, a, b, vec, (bf16_t*)operand, init, total, width);
+  else
+    return TL_ERR_ARG;
   return tl_launch_status();
 }
 

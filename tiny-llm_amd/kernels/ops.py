@@ -1431,12 +1431,13 @@ def delta_prepare(p: torch.Tensor, conv_off: int, b_off: int, a: torch.Tensor, c
                   a_log: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor, saved_off: int,
                   req_of_token: torch.Tensor, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, qn: torch.Tensor,
                   kn: torch.Tensor, vc: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, heads: int,
-                  kv_heads: int, dim: int, vdim: int, taps: int, q_scale: float) -> None:
+                  kv_heads: int, dim: int, vdim: int, taps: int, q_scale: float, decay_per_head: bool = False) -> None:
     """What enters the recurrence, per token and head, in float32: q and k after their causal
     convolution and SiLU as unit vectors (q times q_scale), v after its convolution and SiLU, beta =
-    sigmoid(p[t, b_off + h]) and decay = exp(-exp(a_log[h]) * softplus(a[t, h * dim + i] + dt_bias)).
-    Row t of p holds [q | k | v] from column conv_off on; inputs before a request's first token of the
-    step come from its state row, at saved_off."""
+    sigmoid(p[t, b_off + h]) and decay = exp(-exp(a_log[h]) * softplus(a[t, h * dim + i] + dt_bias)); with
+    decay_per_head `a` and dt_bias hold one number per head (a[t, h], dt_bias[h]) and every channel of the head
+    gets the same decay.  Row t of p holds [q | k | v] from column conv_off on; inputs before a request's first
+    token of the step come from its state row, at saved_off."""
     _dev(p, a, conv_w, a_log, dt_bias, state, req_of_token, cu_seqlens, state_slots, qn, kn, vc, beta, decay)
     check_delta_sizes(heads, kv_heads, dim, vdim, taps)
     _rows_2d(p, "projections")
@@ -1446,8 +1447,9 @@ def delta_prepare(p: torch.Tensor, conv_off: int, b_off: int, a: torch.Tensor, c
     channels = 2 * kv_heads * dim + heads * vdim
     _f32_vec(conv_w, channels * taps, "convolution taps")
     _f32_vec(a_log, heads, "A_log")
-    _f32_vec(dt_bias, heads * dim, "dt_bias")
-    if not (a.dtype == torch.float32 and a.shape[0] == T and a.shape[1] >= heads * dim
+    n_decay = heads if decay_per_head else heads * dim
+    _f32_vec(dt_bias, n_decay, "dt_bias")
+    if not (a.dtype == torch.float32 and a.shape[0] == T and a.shape[1] >= n_decay
             and conv_off >= 0 and conv_off + channels <= p.shape[1] and 0 <= b_off and b_off + heads <= p.shape[1]):
         _fail("delta_prepare: columns do not fit")
     if not (state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
@@ -1461,7 +1463,8 @@ def delta_prepare(p: torch.Tensor, conv_off: int, b_off: int, a: torch.Tensor, c
                                    c_int64(state.stride(0)), c_int64(saved_off), _ptr(req_of_token), _ptr(cu_seqlens),
                                    _ptr(state_slots), _ptr(qn), _ptr(kn), _ptr(vc), _ptr(beta), _ptr(decay), c_int(T),
                                    c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim), c_int(taps),
-                                   c_float(q_scale), c_int(_dt(p)), _stream()), "delta_prepare")
+                                   c_float(q_scale), c_int(1 if decay_per_head else 0), c_int(_dt(p)), _stream()),
+           "delta_prepare")
 
 
 def conv_state_update(p: torch.Tensor, conv_off: int, channels: int, state: torch.Tensor, saved_off: int,
@@ -1507,40 +1510,46 @@ DELTA_DECODE_MAX_VDIM = 256      # a thread per value column in the one-kernel d
 DELTA_DECODE_MAX_TAPS = 4         # and its convolutions' inputs in registers
 
 
-def delta_decode(p: torch.Tensor, conv_off: int, b_off: int, low: torch.Tensor, conv_w: torch.Tensor,
+def delta_decode(p: torch.Tensor, conv_off: int, b_off: int, a: torch.Tensor, gate: torch.Tensor, conv_w: torch.Tensor,
                  a_log: torch.Tensor, dt_bias: torch.Tensor, w_norm: torch.Tensor, state: torch.Tensor,
                  saved_off: int, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, z: torch.Tensor, heads: int,
-                 kv_heads: int, dim: int, vdim: int, taps: int, q_scale: float, eps: float) -> bool:
+                 kv_heads: int, dim: int, vdim: int, taps: int, q_scale: float, eps: float,
+                 decay_per_head: bool = False, gate_kind: str = "sigmoid") -> bool:
     """A decode step of the delta rule in one kernel (every request brings one token; row t of the
-    operands is request t): what `delta_prepare`, `delta_recurrence` and `head_norm_gate` do, with
-    `low` [T, heads * dim + heads * vdim] float32 = [decay | gate] pre-activations.  Returns whether
-    the saved convolution inputs were brought up to date as well (every head has q/k channels of its
-    own); if not, `conv_state_update` has to follow."""
-    _dev(p, low, conv_w, a_log, dt_bias, w_norm, state, cu_seqlens, state_slots, z)
+    operands is request t): what `delta_prepare`, `delta_recurrence` and `head_norm_gate` do, with the decay's
+    pre-activations `a` (float32 [T, heads * dim], or [T, heads] with decay_per_head) and the gate's `gate`
+    (float32 [T, heads * vdim]; both may be views into wider rows), the gate's function "sigmoid" or "silu".
+    Returns whether the saved convolution inputs were brought up to date as well (every head has q/k channels
+    of its own); if not, `conv_state_update` has to follow."""
+    _dev(p, a, gate, conv_w, a_log, dt_bias, w_norm, state, cu_seqlens, state_slots, z)
     check_delta_sizes(heads, kv_heads, dim, vdim, taps)
     _rows_2d(p, "projections")
-    _rows_2d(low, "decay and gate pre-activations")
+    _rows_2d(a, "decay pre-activations")
+    _rows_2d(gate, "gate pre-activations")
+    _need(gate_kind in ("sigmoid", "silu"), f"delta_decode: unknown gate {gate_kind!r}")
+    n_decay = heads if decay_per_head else heads * dim
     _i32(cu_seqlens, state_slots)
     R = state_slots.numel()
     channels = 2 * kv_heads * dim + heads * vdim
     _f32_vec(conv_w, channels * taps, "convolution taps")
     _f32_vec(a_log, heads, "A_log")
-    _f32_vec(dt_bias, heads * dim, "dt_bias")
+    _f32_vec(dt_bias, n_decay, "dt_bias")
     _f32_vec(w_norm, vdim, "the head norm's weight")
-    if not (p.shape[0] == R and low.shape[0] == R and low.dtype == torch.float32
-            and low.shape[1] >= heads * (dim + vdim) and conv_off + channels <= p.shape[1] and b_off + heads <= p.shape[1]
+    if not (p.shape[0] == R and a.shape[0] == R and gate.shape[0] == R and a.dtype == gate.dtype == torch.float32
+            and a.shape[1] >= n_decay and gate.shape[1] >= heads * vdim and conv_off + channels <= p.shape[1] and b_off + heads <= p.shape[1]
             and cu_seqlens.numel() == R + 1 and vdim <= DELTA_DECODE_MAX_VDIM and taps <= DELTA_DECODE_MAX_TAPS
             and vdim % 4 == 0 and state.stride(0) % 4 == 0
             and state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
             and saved_off + channels * (taps - 1) <= state.shape[1] and heads * dim * vdim <= saved_off
-            and z.dtype == p.dtype and z.is_contiguous() and tuple(z.shape) == (R, heads * vdim)):
+            and (z.dtype == p.dtype or p.dtype == torch.float32) and z.is_contiguous() and tuple(z.shape) == (R, heads * vdim)):
         _fail("delta_decode: shapes do not fit (one row per request)")
-    _check(_lib().tl_delta_decode(_ptr(p), c_int64(p.stride(0)), c_int(conv_off), c_int(b_off), _ptr(low),
-                                  c_int64(low.stride(0)), _ptr(conv_w), _ptr(a_log), _ptr(dt_bias), _ptr(w_norm),
+    _check(_lib().tl_delta_decode(_ptr(p), c_int64(p.stride(0)), c_int(conv_off), c_int(b_off), _ptr(a),
+                                  c_int64(a.stride(0)), c_int(1 if decay_per_head else 0), _ptr(gate),
+                                  c_int64(gate.stride(0)), c_int(1 if gate_kind == "silu" else 0), _ptr(conv_w), _ptr(a_log), _ptr(dt_bias), _ptr(w_norm),
                                   _ptr(state), c_int64(state.stride(0)), c_int64(saved_off), _ptr(cu_seqlens),
                                   _ptr(state_slots), _ptr(z), c_int(R), c_int(heads), c_int(kv_heads), c_int(dim),
                                   c_int(vdim), c_int(taps), c_float(q_scale), c_float(eps), c_int(heads == kv_heads),
-                                  c_int(_dt(p)), _stream()),
+                                  c_int(_dt(p)), c_int(_dt(z)), _stream()),
            "delta_decode")
     return heads == kv_heads
 
@@ -1585,6 +1594,38 @@ def layer_norm_sum(y: Optional[torch.Tensor], weight: torch.Tensor, bias: torch.
     _check(_lib().tl_layer_norm_sum(_ptr(y), _ptr(weight), _ptr(bias), _ptr(x), _ptr(copy), c_int(T), c_int(H),
                                     c_float(alpha), c_float(eps), c_int(_dt(copy) if copy is not None else 0), _stream()),
            "layer_norm_sum")
+    return x
+
+
+LAYER_NORM_ADD_MAX = 8192       # widest row `layer_norm_add` keeps in registers (csrc/layer_norm.hip)
+
+
+def layer_norm_add(y: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, x: torch.Tensor, mult: float, eps: float,
+                   then=None) -> torch.Tensor:
+    """x[t] <- x[t] + mult * (LN(y[t]) * weight + bias), in place, float32 (y the sublayer's result, float32 [T, H]).
+    then = (weight2, bias2, eps2, out): out[t] ([T, H] of either element type) also receives LN(x[t]) * weight2 +
+    bias2 of the new rows, in the same kernel."""
+    _dev(y, weight, bias, x)
+    if not (x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous()):
+        _fail("layer_norm_add: the stream is contiguous float32 [T, H]")
+    T, H = x.shape
+    _need(H <= LAYER_NORM_ADD_MAX, f"layer_norm_add: rows of at most {LAYER_NORM_ADD_MAX} elements")
+    if not (y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape) == (T, H)):
+        _fail("layer_norm_add: the sublayer's result is contiguous float32 [T, H]")
+    _f32_vec(weight, H, "the layer norm's weight")
+    _f32_vec(bias, H, "the layer norm's bias")
+    w2 = b2 = out = None
+    eps2 = 0.0
+    if then is not None:
+        w2, b2, eps2, out = then
+        _dev(w2, b2, out)
+        _f32_vec(w2, H, "the next norm's weight")
+        _f32_vec(b2, H, "the next norm's bias")
+        if not (out.is_contiguous() and tuple(out.shape) == (T, H)):
+            _fail("layer_norm_add: the next norm's output is contiguous [T, H]")
+    _check(_lib().tl_layer_norm_add(_ptr(y), _ptr(weight), _ptr(bias), _ptr(x), _ptr(w2), _ptr(b2), _ptr(out), c_int(T),
+                                    c_int(H), c_float(mult), c_float(eps), c_float(eps2),
+                                    c_int(_dt(out) if out is not None else 0), _stream()), "layer_norm_add")
     return x
 
 
@@ -2020,8 +2061,9 @@ MOE_MAX_ROUTED = 1024       # experts the router kernel takes (csrc/moe.hip)
 
 
 def moe_route(z: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, groups: int = 1, keep: int = 1,
-              scale: float = 1.0) -> None:
-    """A router over the logits z (float32 [T, E], rows may be wider apart): scores s = softmax(z) over all experts;
+              scale: float = 1.0, bias: Optional[torch.Tensor] = None) -> None:
+    """A router over the logits z (float32 [T, E], rows may be wider apart; `bias`, float32 [E], is added to every
+    row if given): scores s = softmax(z) over all experts;
     the experts lie in `groups` equal runs of neighbours, a run's score is its largest, and only experts of the
     `keep` best runs may be chosen (groups <= 1: all may); ids[t] (int32 [T, top]) names the `top` largest scores
     among those, largest first (equal scores: the lower index first), and weights[t] (float32 [T, top]) =
@@ -2034,11 +2076,14 @@ def moe_route(z: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, groups:
     _need(ids.dtype == torch.int32 and ids.is_contiguous() and tuple(ids.shape) == (T, top) and top > 0,
           "moe_route: ids are contiguous int32 [T, top]")
     _f32_vec(weights, T * top, "moe_route weights")
+    if bias is not None:
+        _dev(bias)
+        _f32_vec(bias, E, "moe_route bias")
     _need(0 < top <= E <= MOE_MAX_ROUTED, f"moe_route: 1 to {MOE_MAX_ROUTED} experts, top within them")
     if groups > 1:
         _need(E % groups == 0 and 0 < keep <= groups and top <= keep * (E // groups),
               "moe_route: equal groups, 1 to `groups` of them kept, holding at least `top` experts")
-    _check(_lib().tl_moe_route(_ptr(z), c_int64(z.stride(0)), _ptr(ids), _ptr(weights), c_int(T), c_int(E), c_int(top),
+    _check(_lib().tl_moe_route(_ptr(z), c_int64(z.stride(0)), _ptr(bias), _ptr(ids), _ptr(weights), c_int(T), c_int(E), c_int(top),
                                c_int(groups), c_int(keep), c_float(scale), _stream()), "moe_route")
 
 
@@ -2090,3 +2135,122 @@ def embedding_pairs(tokens: torch.Tensor, positions: torch.Tensor, req_of_token:
                                      c_int(H), c_int(V), c_int(pairs.shape[0] - 1), c_int(int(mul_prev)),
                                      c_int(int(mul_cur)), c_float(scale), c_int(_dt(table)), _stream()), "embedding_pairs")
     return out
+
+
+# ------------------------------------------- the general step between the q/k/v product and the attention kernel
+ATTN_PREPARE_MAX_DIM = 256      # numbers a unit (one map of one head) may have, and the padded head size D
+
+
+def attn_prepare(p: torch.Tensor, bias: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], positions: torch.Tensor,
+                 cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
+                 q_out: torch.Tensor, k_caches, v_cache: Optional[torch.Tensor], heads: int, kv_heads: int, maps: int,
+                 dim: int, vdim: int, v_off: int, rot: int = 0, pairing: str = "half", whole_norm: bool = False,
+                 unit_norm: bool = False, eps: float = 1e-6, q_temp=None) -> None:
+    """From the float32 product p [T, >= v_off + kv_heads * vdim] = [q: heads * maps units of dim | k: kv_heads * maps
+    units | v: kv_heads heads of vdim, from column v_off]: bias added (float32 over [q | k | v]), an RMS norm over ALL of
+    a token's q numbers (and all of its k numbers) with weights norm_w (float32 over [q | k], `whole_norm`), the first
+    `rot` dims of every unit rotated by the token's position, every unit divided by its own root mean square
+    (`unit_norm`), queries times 1 + coef * ln(floor((pos + 1) / every) + 1) (`q_temp` = (coef, every)).  Queries leave
+    as q_out [maps, T, heads * D] rounded to the engine's type, keys of map m go to k_caches[m] and values to v_cache
+    (pages [blocks, kv_heads, block, D]) at the tokens' slots; D is q_out's head size, what lies beyond dim or vdim is
+    written as zeros.  slot_mapping None (or a negative slot) stores nothing."""
+    k_caches = tuple(k_caches) if k_caches is not None else ()
+    _dev(p, bias, norm_w, positions, cos, sin, slot_mapping, q_out, v_cache, *k_caches)
+    _rows_2d(p, "attn_prepare input")
+    T = p.shape[0]
+    _need(p.dtype == torch.float32, "attn_prepare: the product is float32")
+    _need(maps in (1, 2) and heads > 0 and kv_heads > 0 and heads % kv_heads == 0, "attn_prepare: one or two maps, heads a "
+          "multiple of kv heads")
+    _need(q_out.dim() == 3 and q_out.is_contiguous() and q_out.shape[0] == maps and q_out.shape[1] == T
+          and q_out.shape[2] % heads == 0, "attn_prepare: queries leave as contiguous [maps, T, heads * D]")
+    D = q_out.shape[2] // heads
+    _need(0 < dim <= D and 0 < vdim <= D and D <= ATTN_PREPARE_MAX_DIM, f"attn_prepare: dim and vdim within D = {D} <= "
+          f"{ATTN_PREPARE_MAX_DIM}")
+    q_size, k_size, v_size = heads * maps * dim, kv_heads * maps * dim, kv_heads * vdim
+    _need(v_off >= q_size + k_size and v_off + v_size <= p.shape[1], "attn_prepare: columns do not fit")
+    if bias is not None:
+        _f32_vec(bias, q_size + k_size + v_size, "attn_prepare bias")
+    if whole_norm:
+        _need(norm_w is not None, "attn_prepare: the norm over the whole projection needs its weights")
+        _f32_vec(norm_w, q_size + k_size, "attn_prepare norm weights")
+    _need(pairing in ROPE_PAIRINGS, f"attn_prepare: rotary pairing {pairing!r} is not built")
+    _need(rot % 2 == 0 and 0 <= rot <= dim, "attn_prepare: the rotated dims are even and within dim")
+    _i32(positions)
+    _need(positions.numel() == T, "attn_prepare: one position per row")
+    if rot:
+        _need(cos is not None and sin is not None and cos.dtype == sin.dtype == torch.float32 and cos.is_contiguous()
+              and sin.is_contiguous() and cos.shape == sin.shape and cos.shape[1] == rot // 2,
+              "attn_prepare: angle tables are float32 [positions, rot / 2]")
+    block_size = 1
+    if slot_mapping is not None:
+        _i32(slot_mapping)
+        _need(slot_mapping.numel() == T and len(k_caches) == maps and v_cache is not None,
+              "attn_prepare: one slot per row, a key cache per map and a value cache")
+        for c in k_caches + (v_cache,):
+            _need(c.dtype == q_out.dtype and c.dim() == 4 and c.is_contiguous() and c.shape[1] == kv_heads
+                  and c.shape[3] == D and c.shape == v_cache.shape, "attn_prepare: caches are contiguous "
+                  "[blocks, kv_heads, block, D] of the queries' type")
+        block_size = v_cache.shape[2]
+    coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp else (0.0, 0)
+    _need(every >= 0, "attn_prepare: the temperature's step is positive")
+    store = slot_mapping is not None
+    _check(_lib().tl_attn_prepare(_ptr(p), c_int64(p.stride(0)), _ptr(bias), _ptr(norm_w), _ptr(positions), _ptr(cos),
+                                  _ptr(sin), _ptr(slot_mapping), _ptr(q_out), c_int64(q_out.stride(1)),
+                                  c_int64(q_out.stride(0)), _ptr(k_caches[0] if store else None),
+                                  _ptr(k_caches[1] if store and maps == 2 else None), _ptr(v_cache if store else None),
+                                  c_int(T), c_int(heads), c_int(kv_heads), c_int(maps), c_int(dim), c_int(vdim), c_int(D),
+                                  c_int(v_off), c_int(rot), c_int(ROPE_PAIRINGS.index(pairing)),
+                                  c_int(1 if whole_norm else 0), c_int(1 if unit_norm else 0), c_float(eps), c_float(coef),
+                                  c_int(every), c_int(block_size), c_int(_dt(q_out)), _stream()), "attn_prepare")
+
+
+ATTN_GATES = {None: 0, "head": 1, "element": 2}
+
+
+def attn_finish(a0: torch.Tensor, a1: Optional[torch.Tensor], gate: Optional[torch.Tensor], z: torch.Tensor, heads: int,
+                vdim: int, lam: float = 0.0, sub_norm: bool = False, eps: float = 1e-6, scale: float = 1.0,
+                gate_kind: Optional[str] = None, tail: int = 0) -> torch.Tensor:
+    """Behind the attention kernel: of every head's D numbers the first vdim, o = a0 - lam * a1 (a1 None: o = a0),
+    divided by the head's root mean square (`sub_norm`), times `scale`, times sigmoid(gate) (float32, one number per
+    token and head for "head", per element [T, heads * vdim] for "element"); z[t] = the heads side by side, then
+    `tail` columns 1, 0, 0, ... (the one meets a bias kept as one more column of the next product's weight)."""
+    _dev(a0, a1, gate, z)
+    _rows_2d(a0, "attn_finish input")
+    _rows_2d(z, "attn_finish output")
+    T = a0.shape[0]
+    _need(a0.shape[1] % heads == 0, "attn_finish: the input is [T, heads * D]")
+    D = a0.shape[1] // heads
+    _need(0 < vdim <= D and vdim <= ATTN_PREPARE_MAX_DIM and z.dtype == a0.dtype and z.shape[0] == T
+          and z.shape[1] == heads * vdim + tail and 0 <= tail <= 64, "attn_finish: z is [T, heads * vdim + tail] of "
+          "the input's type")
+    if a1 is not None:
+        _need(a1.dtype == a0.dtype and a1.shape == a0.shape and a1.stride() == a0.stride(),
+              "attn_finish: the second map has the first one's layout")
+    _need(gate_kind in ATTN_GATES, f"attn_finish: unknown gate {gate_kind!r}")
+    if gate_kind is not None:
+        _rows_2d(gate, "attn_finish gate")
+        _need(gate.dtype == torch.float32 and gate.shape[0] == T
+              and gate.shape[1] == (heads if gate_kind == "head" else heads * vdim), "attn_finish: the gate is float32, "
+              "one number per head or per element")
+    _check(_lib().tl_attn_finish(_ptr(a0), _ptr(a1), c_int64(a0.stride(0)), _ptr(gate if gate_kind else None),
+                                 c_int64(gate.stride(0) if gate_kind else 0), _ptr(z), c_int64(z.stride(0)), c_int(T),
+                                 c_int(heads), c_int(vdim), c_int(D), c_float(lam), c_int(1 if sub_norm else 0),
+                                 c_float(eps), c_float(scale), c_int(ATTN_GATES[gate_kind]), c_int(tail), c_int(_dt(z)),
+                                 _stream()), "attn_finish")
+    return z
+
+
+def stream_join(a: torch.Tensor, b: torch.Tensor, vec: Optional[torch.Tensor], operand: torch.Tensor,
+                init: torch.Tensor) -> None:
+    """operand[t] = [a[t] | b[t]] in operand's element type (a, b float32 [T, W]); init[t] = vec (float32 [W]; zeros
+    without one): the row a product over `operand` then adds its result to."""
+    _dev(a, b, vec, operand, init)
+    T, W = a.shape
+    for t in (a, b, init):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (T, W),
+              "stream_join: streams and the initial rows are contiguous float32 [T, W]")
+    _need(operand.is_contiguous() and tuple(operand.shape) == (T, 2 * W), "stream_join: the operand is contiguous [T, 2W]")
+    if vec is not None:
+        _f32_vec(vec, W, "stream_join vector")
+    _check(_lib().tl_stream_join(_ptr(a), _ptr(b), _ptr(vec), _ptr(operand), _ptr(init), c_int(T), c_int(W),
+                                 c_int(_dt(operand)), _stream()), "stream_join")

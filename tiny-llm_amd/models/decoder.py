@@ -13,6 +13,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ..config.spec import LayerSpec, ModelSpec, PartSpec
+from ..kernels import ops
 from ..parts import BLOCKS, REGISTRIES, CacheSpec, LayerCache, Part, StateSpec, WeightSpec
 
 TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
@@ -63,6 +64,8 @@ class Decoder:
         self.device = torch.device(device)
         self.embedding = build_part("embedding", spec.embedding, spec.embedding.name, self.dtype, self.device)
         self.layers: List[Layer] = [Layer(ls, self.dtype, self.device) for ls in spec.layers]
+        self.stream_parts: List[Part] = [build_part("stream", ps, ps.name, self.dtype, self.device)
+                                         for ps in spec.stream_parts]
         self.final_norm = build_part("norm", spec.final_norm, spec.final_norm.name, self.dtype, self.device)
         self.lm_head = build_part("head", spec.lm_head, spec.lm_head.name, self.dtype, self.device)
         # cache and state views by role, per plan entry; attached by the runner once the pools exist
@@ -77,6 +80,7 @@ class Decoder:
         out = [self.embedding]
         for l in self.layers:
             out.extend(l.parts())
+        out.extend(self.stream_parts)
         out.extend([self.final_norm, self.lm_head])
         return out
 
@@ -147,7 +151,10 @@ class Decoder:
         elif stage == self.num_stages - 1:
             parts = [self.final_norm, self.lm_head]
         else:
-            parts = self.layers[self.spec.plan[stage - 1].layer].parts()
+            entry = self.spec.plan[stage - 1]
+            parts = self.layers[entry.layer].parts()
+            if entry.before is not None:
+                parts = parts + [self.stream_parts[entry.before[0]]]
         parts = parts + [getattr(p, "position", None) for p in parts]
         return all(p.graph_safe for p in parts if p is not None)
 
@@ -183,18 +190,34 @@ class Decoder:
                 x = self.embedding.forward(ctx.tokens, ctx, state=self.embedding_state)
             else:
                 x = self.embedding.forward(ctx.tokens, ctx)
+        # A model with parts that act on the stream between layer runs keeps the embedding's output of the step for
+        # them: in a buffer by name, so that a later call for the same step finds it.  The stream then goes on in a
+        # buffer of its own (by a copy here if layers run ahead of the first such part, else that part moves it).
+        origin = None
+        if self.stream_parts:
+            if first == 0:
+                origin = x
+                if plan[0].before is None:
+                    x = ops.cast_rows(origin, ops.scratch("loop_stream", x.shape, torch.float32, x.device))
+            else:
+                origin = ops.scratch("residual", x.shape, torch.float32, x.device)
         # A block may prepare the norm that reads its result (the next block's first norm, or the
         # final norm) in its last product; `prepared` carries that from one block to the next.
         prepared = None
         for st in range(max(first, 1), min(last, n - 1)):
             i = st - 1
             block = self.layers[plan[i].layer].block
+            if plan[i].before is not None:
+                part, turn = plan[i].before
+                x, prepared = self.stream_parts[part].forward(x, origin, ctx, turn), None
             if not hasattr(block, "forward_chained"):
                 x, prepared = block.forward(x, ctx, self.caches[i], self.states[i]), None
                 continue
             next_norm = None
             if st + 1 < last:                    # what reads this block's result runs in this call
-                if i + 1 < len(plan):
+                if i + 1 < len(plan) and plan[i + 1].before is not None:
+                    next_norm = None             # a stream part stands between: it reads the stream itself
+                elif i + 1 < len(plan):
                     nxt = self.layers[plan[i + 1].layer].block
                     next_norm = getattr(nxt, "first_norm", None) if hasattr(nxt, "forward_chained") else None
                 else:

@@ -173,6 +173,15 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class StreamPart(Part):
+    """A part that acts on the residual stream between two layer runs: `forward(x, origin, ctx, turn)` returns the
+    new stream (float32 [T, hidden]; it may write into x but not into origin).  `origin` is the embedding's output
+    of this step, `turn` the number the plan gives (which pass through a repeated run of layers begins)."""
+
+    def forward(self, x: torch.Tensor, origin: torch.Tensor, ctx, turn: int) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class ChannelScale(Part):
     """One learned factor per channel (a sublayer's result times a vector)."""
 
@@ -254,12 +263,14 @@ MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 POSITION_ENCODINGS = Registry("position encoding")
 SCALES = Registry("channel scale")
+STREAM_PARTS = Registry("stream part")
 BLOCKS = Registry("block arrangement")
 
 
 # a block's roles and the model's own parts name their registry by these keys
 REGISTRIES = {"embedding": EMBEDDINGS, "head": HEADS, "norm": NORMS, "mixer": MIXERS,
-              "feed_forward": FEED_FORWARDS, "position_encoding": POSITION_ENCODINGS, "scale": SCALES}
+              "feed_forward": FEED_FORWARDS, "position_encoding": POSITION_ENCODINGS, "scale": SCALES,
+              "stream": STREAM_PARTS}
 
 
 def register_embedding(name, factory, **kw): EMBEDDINGS.register(name, factory, **kw)
@@ -269,4 +280,5 @@ def register_mixer(name, factory, **kw): MIXERS.register(name, factory, **kw)
 def register_feed_forward(name, factory, **kw): FEED_FORWARDS.register(name, factory, **kw)
 def register_position_encoding(name, factory, **kw): POSITION_ENCODINGS.register(name, factory, **kw)
 def register_scale(name, factory, **kw): SCALES.register(name, factory, **kw)
+def register_stream_part(name, factory, **kw): STREAM_PARTS.register(name, factory, **kw)
 def register_block(name, factory, **kw): BLOCKS.register(name, factory, **kw)

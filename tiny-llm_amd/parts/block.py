@@ -2,7 +2,9 @@
 x + ffn(norm(x)) (tiny_llm/parser/llama_parser.cpp:194-255).  "output_norm" puts the norm on each
 sublayer's result instead: x + scale * norm(mixer(x)), then x + scale * norm(ffn(x)); the
 sublayers read the residual stream itself.  "sum_norm" puts the norm behind the sum:
-x <- norm(alpha * x + mixer(x)), then x <- norm(alpha * x + ffn(x)), alpha a constant of the model."""
+x <- norm(alpha * x + mixer(x)), then x <- norm(alpha * x + ffn(x)), alpha a constant of the model.
+"sandwich" has a norm in front of and behind every sublayer: x <- x + mult * norm_b(mixer(norm_a(x))), then
+x <- x + mult * norm_d(ffn(norm_c(x))), mult a constant of the model."""
 from __future__ import annotations
 
 import torch
@@ -164,6 +166,72 @@ class SumNormBlock(Block):
         return x, copy
 
 
+class NormedRows:
+    """What a sandwich block hands to the block behind it: the stream as that block's first norm sees it,
+    formed by the kernel that wrote the stream."""
+
+    def __init__(self, norm, rows: torch.Tensor):
+        self.norm, self.rows = norm, rows
+
+
+class SandwichBlock(Block):
+    """x <- x + mult * LNb(mixer(LNa(x))); x <- x + mult * LNd(ffn(LNc(x))): a norm in front of and behind every
+    sublayer.  The sublayers are called with `residual=None` and return their result by itself in float32; the norm
+    behind a sublayer, the scaled sum and the norm in front of whatever reads the stream next (this block's
+    feed-forward, or the next block's mixer if that block says which norm it begins with) are ONE kernel.  A layer
+    may have no feed-forward (and then neither of its norms)."""
+    roles = {"mixer_norm": "norm", "mixer": "mixer", "mixer_out_norm": "norm",
+             "ffn_norm": "norm", "ffn": "feed_forward", "ffn_out_norm": "norm"}
+    optional = ("ffn_norm", "ffn", "ffn_out_norm")
+
+    def __init__(self, parts, mult: float = 1.0):
+        super().__init__(parts)
+        self.mult = float(mult)
+        self.mixer_norm, self.mixer, self.mixer_out_norm = parts["mixer_norm"], parts["mixer"], parts["mixer_out_norm"]
+        self.ffn_norm, self.ffn, self.ffn_out_norm = parts.get("ffn_norm"), parts.get("ffn"), parts.get("ffn_out_norm")
+        if len({self.ffn is None, self.ffn_norm is None, self.ffn_out_norm is None}) != 1:
+            raise ValueError("sandwich: a feed-forward comes with both of its norms, and they with a feed-forward")
+        for n in (self.mixer_out_norm, self.ffn_out_norm):
+            if n is not None and not hasattr(n, "add_scaled_norm"):
+                raise ValueError(f"sandwich: the norm {type(n).__name__} cannot sit on a sublayer's result (no add_scaled_norm)")
+
+    @property
+    def first_norm(self):
+        """The norm that reads this block's input, for whoever writes that input."""
+        return self.mixer_norm
+
+    def forward(self, x, ctx, caches, states):
+        return self.forward_chained(x, ctx, caches, states)[0]
+
+    @staticmethod
+    def _fusable(out_norm, next_norm):
+        """Whether `out_norm.add_scaled_norm` can also produce `next_norm` of the new stream."""
+        return type(next_norm) is type(out_norm) and getattr(next_norm, "hidden_size", None) == out_norm.hidden_size
+
+    def forward_chained(self, x, ctx, caches, states, prepared=None, next_norm=None):
+        """`prepared`: NormedRows of this block's first norm if the block in front formed them; returned likewise
+        for the block behind when `next_norm` is a norm this block's last kernel can form."""
+        if isinstance(prepared, NormedRows) and prepared.norm is self.mixer_norm:
+            h = prepared.rows
+        else:
+            h = self.mixer_norm.forward(x)
+        y = self.mixer.forward(h, ctx, caches.get("mixer"), states.get("mixer"), None)
+        if self.ffn is None:
+            return x, self._add(self.mixer_out_norm, y, x, next_norm)
+        handed = self._add(self.mixer_out_norm, y, x, self.ffn_norm)
+        h = handed.rows if handed is not None else self.ffn_norm.forward(x)
+        y = self.ffn.forward(h, ctx, None)
+        return x, self._add(self.ffn_out_norm, y, x, next_norm)
+
+    def _add(self, out_norm, y, x, next_norm):
+        if next_norm is not None and self._fusable(out_norm, next_norm):
+            rows = out_norm.add_scaled_norm(y, x, self.mult, then=next_norm)
+            return NormedRows(next_norm, rows) if rows is not None else None
+        out_norm.add_scaled_norm(y, x, self.mult)
+        return None
+
+
 register_block("pre_norm", PreNormBlock)
+register_block("sandwich", SandwichBlock)
 register_block("sum_norm", SumNormBlock)
 register_block("output_norm", OutputNormBlock)

@@ -80,11 +80,12 @@ class LMHead(Head):
     accepts_lazy_norm = True
 
     def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int, tied_to: str = None,
-                 weight_name: str = "weight", softcap: float = 0.0):
+                 weight_name: str = "weight", softcap: float = 0.0, tied_exact: bool = False):
         """softcap c > 0: logits <- c * tanh(logits / c)."""
         super().__init__(prefix, dtype, device)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.tied_to = tied_to          # weight prefix of the embedding whose table this head shares
+        self.tied_exact = bool(tied_exact)
         self.tensor_name = f"{prefix}.{weight_name}" if weight_name else prefix
         self.softcap = float(softcap or 0.0)
         if self.softcap < 0:
@@ -93,7 +94,11 @@ class LMHead(Head):
         self.weight: Optional[torch.Tensor] = None
 
     def weights(self) -> List[WeightSpec]:
-        alias = f"{self.tied_to}.weight" if self.tied_to else None
+        # `tied_to` names the embedding's weight prefix (its table is `<prefix>.weight`), or, with a name that the
+        # checkpoint holds as it stands (an embedding whose prefix IS the tensor), that tensor
+        alias = None
+        if self.tied_to:
+            alias = self.tied_to if self.tied_exact else f"{self.tied_to}.weight"
         return [WeightSpec(self.tensor_name, (self.vocab_size, self.hidden_size), alias_of=alias)]
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:

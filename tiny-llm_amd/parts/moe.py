@@ -13,7 +13,10 @@ Tensor names below the prefix: e<i>.gate|up|down, table, shared.gate|up|down, sh
 over all experts (float32); the experts lie in `groups` equal runs of neighbours, a run's score is its largest
 score and only experts of the `keep` best runs may be chosen; the `top` largest scores among those are chosen and
 weigh s_j / (sum of the chosen + 1e-20) * scale; an optional shared expert of the same form runs for every token
-and is added.  Tensor names below the prefix: e<i>.up|down, router, shared.up|down.
+and is added.  Tensor names below the prefix: e<i>.up|down, router, shared.up|down.  Options: `activation="swiglu"`
+makes the experts gated units down(silu(gate(h)) * up(h)) (tensors e<i>.gate|up|down); `router_bias` adds a bias per
+expert to the router's logits (tensor router<bias_suffix>).  With one group and scale 1 the weights are the softmax
+over the chosen logits alone: exp(z_j) / sum over the chosen of exp(z_i), whatever the other experts' logits are.
 """
 from __future__ import annotations
 
@@ -139,7 +142,7 @@ class RoutedMoE(FeedForward):
 
     def __init__(self, prefix, dtype, device, *, hidden_size: int, num_experts: int, top: int, intermediate_size: int,
                  groups: int = 1, keep: int = 1, scale: float = 1.0, activation: str = "relu2",
-                 shared: Optional[dict] = None):
+                 shared: Optional[dict] = None, router_bias: bool = False, bias_suffix: str = ".b"):
         """shared: None, or {"intermediate_size": F} (optionally "activation") for the shared expert."""
         super().__init__(prefix, dtype, device)
         self.hidden_size, self.num_experts, self.top = int(hidden_size), int(num_experts), int(top)
@@ -152,9 +155,12 @@ class RoutedMoE(FeedForward):
                                 or self.top > self.keep * (self.num_experts // self.groups)):
             raise ValueError(f"{prefix}: {self.num_experts} experts in {self.groups} groups of which {self.keep} are "
                              f"kept: groups must be equal and the kept ones hold at least top = {self.top} experts")
-        if activation not in ops.MOE_ACTIVATIONS or activation is None:
-            raise ValueError(f"{prefix}: activation {activation!r} is not built; known: relu2")
+        self.gated = activation == "swiglu"
+        if not self.gated and (activation not in ops.MOE_ACTIVATIONS or activation is None):
+            raise ValueError(f"{prefix}: activation {activation!r} is not built; known: relu2, swiglu")
         self.activation = activation
+        self.router_bias, self.bias_suffix = bool(router_bias), bias_suffix
+        self.b_router = None
         ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
         ops.check_linear_sizes(dtype, self.intermediate_size, f"{prefix}: expert intermediate_size")
         self.shared = None
@@ -168,17 +174,27 @@ class RoutedMoE(FeedForward):
         p, W, F = self.prefix, self.hidden_size, self.intermediate_size
         out = []
         for e in range(self.num_experts):
+            if self.gated:
+                out.append(WeightSpec(f"{p}.e{e}.gate", (F, W)))
             out += [WeightSpec(f"{p}.e{e}.up", (F, W)), WeightSpec(f"{p}.e{e}.down", (W, F))]
         out.append(WeightSpec(f"{p}.router", (self.num_experts, W)))
+        if self.router_bias:
+            out.append(WeightSpec(f"{p}.router{self.bias_suffix}", (self.num_experts,), role="vector", init="zeros"))
         if self.shared is not None:
             out += self.shared.weights()
         return out
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         p, E = self.prefix, self.num_experts
-        self.w_up = torch.stack([tensors[f"{p}.e{e}.up"] for e in range(E)]).contiguous()
+        if self.gated:      # an expert's first product gives [gate | up]
+            self.w_up = torch.stack([torch.cat([tensors[f"{p}.e{e}.gate"], tensors[f"{p}.e{e}.up"]], dim=0)
+                                     for e in range(E)]).contiguous()
+        else:
+            self.w_up = torch.stack([tensors[f"{p}.e{e}.up"] for e in range(E)]).contiguous()
         self.w_down = torch.stack([tensors[f"{p}.e{e}.down"] for e in range(E)]).contiguous()
         self.w_router = tensors[f"{p}.router"].contiguous()
+        if self.router_bias:
+            self.b_router = tensors[f"{p}.router{self.bias_suffix}"].to(torch.float32).contiguous()
         if self.shared is not None:
             self.shared.bind(tensors)
             # one product reads h for the router's logits and the shared expert's hidden units (float32 out):
@@ -201,7 +217,7 @@ class RoutedMoE(FeedForward):
             Fs = self.shared.intermediate_size
             first = ops.scratch("moe_first", (T, self.shared_off + Fs), torch.float32, dev)
             ops.linear(h, self.w_first, first)
-            ops.moe_route(first[:, :E], ids, wts, self.groups, self.keep, self.scale)
+            ops.moe_route(first[:, :E], ids, wts, self.groups, self.keep, self.scale, self.b_router)
             zs = ops.activate_rows(first[:, self.shared_off:], ops.scratch("ffn_gated", (T, Fs), self.dtype, dev),
                                    self.shared.activation)
             if residual is None:
@@ -211,7 +227,7 @@ class RoutedMoE(FeedForward):
         else:
             logits = ops.scratch("moe_router", (T, E), torch.float32, dev)
             ops.linear(h, self.w_router, logits)
-            ops.moe_route(logits, ids, wts, self.groups, self.keep, self.scale)
+            ops.moe_route(logits, ids, wts, self.groups, self.keep, self.scale, self.b_router)
             base = residual                     # the experts are added to the stream itself (or stand alone)
         rows = T * top
         out = base if base is not None else ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev)
@@ -226,19 +242,31 @@ class RoutedMoE(FeedForward):
             hp = ops.scratch("moe_rows_in", (cap, self.hidden_size), self.dtype, dev)
             pos = ops.scratch("moe_row_pos", (rows,), torch.int32, dev)
             ops.moe_gather(h, top, plan, rows, E, R, hp, pos)
-            up = ops.scratch("moe_up", (cap, F), torch.float32, dev)        # float32: rounded once, behind the activation
-            ops.linear_grouped(hp, self.w_up, runs, up)
-            z = ops.activate_rows(up, ops.scratch("moe_gated", (cap, F), self.dtype, dev), self.activation)
+            z = ops.scratch("moe_gated", (cap, F), self.dtype, dev)
+            if self.gated:
+                gup = ops.scratch("moe_gate_up", (cap, 2 * F), self.dtype, dev)
+                ops.linear_grouped(hp, self.w_up, runs, gup)
+                ops.silu_mul(gup, z)
+            else:
+                up = ops.scratch("moe_up", (cap, F), torch.float32, dev)        # float32: rounded once, behind the activation
+                ops.linear_grouped(hp, self.w_up, runs, up)
+                ops.activate_rows(up, z, self.activation)
             y = ops.scratch("moe_rows_out", (cap, self.hidden_size), torch.float32, dev)
             ops.linear_grouped(z, self.w_down, runs, y)
             ops.moe_combine_at(y, pos, out, top, 1.0, base, None, wts)
         elif self.dtype == torch.bfloat16 and rows >= self.GROUPED_ROWS:
             # many rows: sorted by expert on the device, tiles of one expert's rows on the matrix cores
-            up = ops.scratch("moe_up", (rows, F), torch.float32, dev)
             plan = ops.scratch("moe_plan", (ops.moe_plan_ints(rows, E),), torch.int32, dev)
             ops.moe_plan(None, ids, plan, E, num_tokens=T)
-            ops.grouped_rows_gemm(h, top, self.w_up, plan, up)
-            z = ops.activate_rows(up, ops.scratch("moe_gated", (rows, F), self.dtype, dev), self.activation)
+            z = ops.scratch("moe_gated", (rows, F), self.dtype, dev)
+            if self.gated:
+                gup = ops.scratch("moe_gate_up", (rows, 2 * F), self.dtype, dev)
+                ops.grouped_rows_gemm(h, top, self.w_up, plan, gup)
+                ops.silu_mul(gup, z)
+            else:
+                up = ops.scratch("moe_up", (rows, F), torch.float32, dev)
+                ops.grouped_rows_gemm(h, top, self.w_up, plan, up)
+                ops.activate_rows(up, z, self.activation)
             y = ops.scratch("moe_rows_out", (rows, self.hidden_size), torch.float32, dev)
             ops.grouped_rows_gemm(z, 1, self.w_down, plan, y)
             ops.moe_combine(y, out, top, 1.0, base, None, wts)
@@ -246,7 +274,12 @@ class RoutedMoE(FeedForward):
             # few rows (decoding) and float32: each row against its own expert's weights, the activation in
             # the first product's kernel
             z = ops.scratch("moe_gated", (rows, F), self.dtype, dev)
-            ops.table_moe_up(h, self.w_up, None, ids, z, self.activation)
+            if self.gated:
+                gup = ops.scratch("moe_gate_up", (rows, 2 * F), self.dtype, dev)
+                ops.table_moe_up(h, self.w_up, None, ids, gup, None)
+                ops.silu_mul(gup, z)
+            else:
+                ops.table_moe_up(h, self.w_up, None, ids, z, self.activation)
             ops.table_moe_down(z, self.w_down, None, ids, out, 1.0, base, None, wts)
         return out
 

@@ -118,7 +118,8 @@ class RMSNorm(Norm):
 class LayerNorm(Norm):
     """(x - mean) / sqrt(var + eps) * w + b over a row, var the mean squared deviation; statistics, weight
     and bias in float32.  `weight_name` / `bias_name`: the tensors' names below the prefix ("" for the
-    prefix itself).  `sum_normed` serves a layer whose norm FOLLOWS the sum: x <- LN(alpha * x + y)."""
+    prefix itself).  `sum_normed` serves a layer whose norm FOLLOWS the sum: x <- LN(alpha * x + y); `add_scaled_norm` one
+    whose norm sits on the sublayer's result: x <- x + mult * LN(y)."""
     graph_safe = True
 
     def __init__(self, prefix, dtype, device, *, hidden_size: int, eps: float, weight_name: str = "weight",
@@ -148,6 +149,19 @@ class LayerNorm(Norm):
         """x <- LN(alpha * x + y) in place (y float32 or None, one kernel); `copy` receives the new x in
         its own element type."""
         return ops.layer_norm_sum(y, self.weight, self.bias, x, alpha, self.eps, copy)
+
+    def add_scaled_norm(self, y: torch.Tensor, x: torch.Tensor, mult: float = 1.0, then: "LayerNorm" = None):
+        """x <- x + mult * LN(y) in place, for a norm that sits on a sublayer's result (y float32, one kernel).
+        `then`: the layer norm that reads the new x next; its result comes out of the same kernel and is returned
+        (None without one, or where the kernel does not take the width)."""
+        if self.hidden_size > ops.LAYER_NORM_ADD_MAX:
+            raise ValueError(f"{self.prefix}: a layer norm behind a sublayer takes rows of at most {ops.LAYER_NORM_ADD_MAX}")
+        if then is None:
+            ops.layer_norm_add(y, self.weight, self.bias, x, mult, self.eps)
+            return None
+        out = ops.scratch("normed", x.shape, then.dtype, x.device, rotate=2)
+        ops.layer_norm_add(y, self.weight, self.bias, x, mult, self.eps, then=(then.weight, then.bias, then.eps, out))
+        return out
 
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         n = x.shape[0] if rows is None else rows.numel()
