@@ -215,8 +215,11 @@ def run_order(cfg):
     return order + [(i, None, False) for i in range(loop["stop"], n)]
 
 
-def forward(cfg, weights, tokens, dtype=torch.float64, trace: Optional[List[torch.Tensor]] = None):
-    """Logits [T, vocab] of one sequence; `trace` collects the residual stream after every layer run."""
+def forward(cfg, weights, tokens, dtype=torch.float64, trace: Optional[List[torch.Tensor]] = None, round_inputs=None):
+    """Logits [T, vocab] of one sequence; `trace` collects the residual stream after every layer run.
+    round_inputs (a torch dtype): every sublayer's normed input is rounded to it and back, the one rounding that
+    any engine with products in that type must make; what it does to the logits says how far two correct
+    implementations in that type may lie apart."""
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     eps, m = cfg["norm"]["eps"], cfg.get("residual_mult", 1.0)
     positions = torch.arange(len(tokens))
@@ -227,10 +230,11 @@ def forward(cfg, weights, tokens, dtype=torch.float64, trace: Optional[List[torc
             x = torch.cat([x, x0], dim=-1) @ w["loop.in"].T + w["loop.step"][t]
         layer, p = cfg["layers"][i], f"l{i}."
         ln = lambda name, y: layer_norm(y, w[p + name], w[p + name + ".b"], eps)
-        y = MIXERS[layer["type"]](ln("norm1", x), sub(w, p + "mix."), layer["mixer"], eps, positions)
+        cut = (lambda h: h.to(round_inputs).to(dtype)) if round_inputs is not None else (lambda h: h)
+        y = MIXERS[layer["type"]](cut(ln("norm1", x)), sub(w, p + "mix."), layer["mixer"], eps, positions)
         x = x + m * ln("norm1b", y)
         if layer.get("mlp"):
-            y = moe(ln("norm2", x), sub(w, p + "mlp."), layer["mlp"])
+            y = moe(cut(ln("norm2", x)), sub(w, p + "mlp."), layer["mlp"])
             x = x + m * ln("norm2b", y)
         if trace is not None:
             trace.append(x.clone())

@@ -30,6 +30,17 @@ __device__ __forceinline__ int first_visible_key(int pos, int window) {
   return 0;
 }
 
+// The `sink` argument of every entry point and kernel here is a set of flags: bit 0, the softmax's denominator has
+// one more term (the sink); bit 1 (the general kernel and the bfloat16 kernels), the result leaves as float32
+// whatever the type of queries and cache (`out` then points to floats, out_stride counts floats): for a caller
+// that goes on in float32 with it (a difference of two maps, a norm per head).
+constexpr int kFlagSink = 1, kFlagOutF32 = 2;
+template <typename T>
+__device__ __forceinline__ void store_result(T* out, int64_t at, float v, int flags) {
+  if (flags & kFlagOutF32) reinterpret_cast<float*>(out)[at] = v;
+  else out[at] = from_f32<T>(v);
+}
+
 constexpr int kMaxHd = 256;
 constexpr int kDPL = kMaxHd / TL_WAVE;  // output dims per lane
 
@@ -92,12 +103,12 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
     m = m_new;
   }
   // a sink: one more term in the denominator, exp(0 - m) in the scores' own scale, that carries no value
-  if (sink) l += expf(-m);
-  T* orow = out + (int64_t)t * out_stride + (int64_t)h * hd;
+  if (sink & kFlagSink) l += expf(-m);
+  const int64_t orow = (int64_t)t * out_stride + (int64_t)h * hd;
 #pragma unroll
   for (int i = 0; i < kDPL; ++i) {
     const int d = lane + i * TL_WAVE;
-    if (d < hd) orow[d] = from_f32<T>(o[i] / l);
+    if (d < hd) store_result(out, orow + d, o[i] / l, sink);
   }
 }
 
@@ -131,7 +142,7 @@ constexpr float kNegBig = -1.0e30f;   // "no key yet": finite, so exp2(m - m') n
 // exp2(s - m) over the keys, m in units of log2 e; the term is exp2(0 - m) (infinite for a very negative m,
 // which makes the result the zero it then is).
 __device__ __forceinline__ float with_sink(float l, float m, int sink) {
-  return sink ? l + __builtin_amdgcn_exp2f(-m) : l;
+  return (sink & kFlagSink) ? l + __builtin_amdgcn_exp2f(-m) : l;
 }
 
 // Two probabilities as two bfloat16 terms each, p = hi + lo, packed pairwise.  hi is p with the low
@@ -538,7 +549,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
     }
     if (n_splits == 1) {
       const float Ls = with_sink(L, M, sink);
-      out[(int64_t)t * out_stride + (int64_t)h * HD + d] = (bf16_t)(Ls > 0.f ? acc / Ls : 0.f);
+      store_result(out, (int64_t)t * out_stride + (int64_t)h * HD + d, Ls > 0.f ? acc / Ls : 0.f, sink);
     } else {
       part_o[(((int64_t)split * n_tokens + t) * nq + h) * HD + d] = acc;
       if (d == 0) {
@@ -1260,7 +1271,19 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
     }
     const float ls = with_sink(l, m_run[rt], sink);
     const float inv = ls > 0.f ? 1.f / ls : 0.f;
-    bf16_t* orow = out + (int64_t)tok[rt] * out_stride + (int64_t)head * HD + g * 4;
+    const int64_t oat = (int64_t)tok[rt] * out_stride + (int64_t)head * HD + g * 4;
+    if (sink & kFlagOutF32) {
+      float* orow = reinterpret_cast<float*>(out) + oat;
+#pragma unroll
+      for (int dt = 0; dt < HDT; ++dt) {
+        f32x4 v4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v4[r] = o[rt][dt][r] * inv;
+        *(f32x4*)(orow + dt * 16) = v4;
+      }
+      continue;
+    }
+    bf16_t* orow = out + oat;
 #pragma unroll
     for (int dt = 0; dt < HDT; ++dt) {
       bf16x4 v4;
@@ -1308,7 +1331,7 @@ __global__ __launch_bounds__(TL_WAVE) void flash_combine_kernel(const float* __r
         }
       }
       const float Ls = with_sink(L, M, sink);
-      out[(int64_t)t * out_stride + (int64_t)h * hd + d] = (bf16_t)(Ls > 0.f ? acc / Ls : 0.f);
+      store_result(out, (int64_t)t * out_stride + (int64_t)h * hd + d, Ls > 0.f ? acc / Ls : 0.f, sink);
     }
     return;
   }
@@ -1340,7 +1363,7 @@ __global__ __launch_bounds__(TL_WAVE) void flash_combine_kernel(const float* __r
       }
     }
     const float Ls = with_sink(L, M, sink);
-    out[(int64_t)t * out_stride + (int64_t)h * hd + d] = (bf16_t)(Ls > 0.f ? acc / Ls : 0.f);
+    store_result(out, (int64_t)t * out_stride + (int64_t)h * hd + d, Ls > 0.f ? acc / Ls : 0.f, sink);
   }
 }
 

@@ -219,15 +219,15 @@ __global__ __launch_bounds__(kPrepThreads) void attn_prepare_kernel(
 //   o <- o * scale * gate,  gate = 1, sigmoid(g[t, head]) (gate_kind 1) or sigmoid(g[t, head * vdim + j]) (2)
 // written side by side as z[t, head * vdim + j]; columns heads * vdim .. heads * vdim + tail - 1 of z become
 // 1, 0, 0, ...: the one meets a bias stored as one more column of the output product's weight.
-template <typename T>
-__global__ __launch_bounds__(TL_WAVE) void attn_finish_kernel(const T* __restrict__ a0, const T* __restrict__ a1,
+template <typename TA, typename T>
+__global__ __launch_bounds__(TL_WAVE) void attn_finish_kernel(const TA* __restrict__ a0, const TA* __restrict__ a1,
                                                               int64_t a_stride, const float* __restrict__ g,
                                                               int64_t g_stride, T* __restrict__ z, int64_t z_stride,
                                                               int heads, int vdim, int D, float lambda, int sub_norm,
                                                               float eps, float scale, int gate_kind, int tail) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const T* s0 = a0 + (int64_t)t * a_stride + (int64_t)h * D;
-  const T* s1 = a1 ? a1 + (int64_t)t * a_stride + (int64_t)h * D : nullptr;
+  const TA* s0 = a0 + (int64_t)t * a_stride + (int64_t)h * D;
+  const TA* s1 = a1 ? a1 + (int64_t)t * a_stride + (int64_t)h * D : nullptr;
   constexpr int kPer = 4;       // heads of up to 256 values
   float o[kPer];
   float ss = 0.f;
@@ -340,24 +340,24 @@ int tl_attn_prepare(const float* p, int64_t p_stride, const float* bias, const f
   return tl_launch_status();
 }
 
-// a0, a1 (a1 null for one map): [n_tokens, heads * D] of the engine's type, rows a_stride apart; g: float32 gates or
-// null; z: [n_tokens, >= heads * vdim + tail], rows z_stride apart.
+// a0, a1 (a1 null for one map): [n_tokens, heads * D] in a_dtype (float32, or z's type), rows a_stride apart; g:
+// float32 gates or null; z: [n_tokens, >= heads * vdim + tail] in dtype, rows z_stride apart.
 int tl_attn_finish(const void* a0, const void* a1, int64_t a_stride, const float* g, int64_t g_stride, void* z,
                    int64_t z_stride, int n_tokens, int heads, int vdim, int D, float lambda, int sub_norm, float eps,
-                   float scale, int gate_kind, int tail, int dtype, hipStream_t stream) {
+                   float scale, int gate_kind, int tail, int a_dtype, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (heads <= 0 || heads > 65535 || vdim <= 0 || D < vdim || vdim > 4 * TL_WAVE || !a0 || !z || gate_kind < 0 ||
       gate_kind > 2 || (gate_kind && !g) || tail < 0 || tail > TL_WAVE)
     return TL_ERR_ARG;
   dim3 grid(n_tokens, heads), b(TL_WAVE);
-  if (dtype == 0)
-    hipLaunchKernelGGL(attn_finish_kernel<float>, grid, b, 0, stream, (const float*)a0, (const float*)a1, a_stride, g,
-                       g_stride, (float*)z, z_stride, heads, vdim, D, lambda, sub_norm, eps, scale, gate_kind, tail);
-  else if (dtype == 1)
-    hipLaunchKernelGGL(attn_finish_kernel<bf16_t>, grid, b, 0, stream, (const bf16_t*)a0, (const bf16_t*)a1, a_stride, g,
-                       g_stride, (bf16_t*)z, z_stride, heads, vdim, D, lambda, sub_norm, eps, scale, gate_kind, tail);
-  else
-    return TL_ERR_ARG;
+#define TL_FINISH(TA, TZ)                                                                                             \
+  hipLaunchKernelGGL((attn_finish_kernel<TA, TZ>), grid, b, 0, stream, (const TA*)a0, (const TA*)a1, a_stride, g,       \
+                     g_stride, (TZ*)z, z_stride, heads, vdim, D, lambda, sub_norm, eps, scale, gate_kind, tail)
+  if (a_dtype == 0 && dtype == 0) TL_FINISH(float, float);
+  else if (a_dtype == 0 && dtype == 1) TL_FINISH(float, bf16_t);
+  else if (a_dtype == 1 && dtype == 1) TL_FINISH(bf16_t, bf16_t);
+  else return TL_ERR_ARG;
+#undef TL_FINISH
   return tl_launch_status();
 }
 

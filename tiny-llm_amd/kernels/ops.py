@@ -601,6 +601,16 @@ def rope_store(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[torch.T
 ROPE_PAIRINGS = ("half", "interleaved")     # the rotation kernel's pairings, by the number it takes
 
 
+def _attn_flags(sink: bool, q: torch.Tensor, out: torch.Tensor) -> int:
+    """The flags the attention kernels take in their `sink` argument: bit 0 the sink term, bit 1 a float32 result
+    from operands of another type (the general kernel and the bfloat16 kernels)."""
+    return (1 if sink else 0) | (2 if (out.dtype == torch.float32 and q.dtype != torch.float32) else 0)
+
+
+def _attn_types_ok(q, k_cache, v_cache, out) -> bool:
+    return q.dtype == k_cache.dtype == v_cache.dtype and out.dtype in (q.dtype, torch.float32)
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     block_tables: torch.Tensor, req_of_token: torch.Tensor, positions: torch.Tensor,
                     out: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, scale: float,
@@ -614,8 +624,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     T = q.shape[0]
     if not (q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim)):
         _fail("q and the attention output must be [T, heads * head_dim]")
-    if not (q.dtype == k_cache.dtype == v_cache.dtype == out.dtype):
-        _fail("q, caches and output must share an element type")
+    if not _attn_types_ok(q, k_cache, v_cache, out):
+        _fail("q and caches must share an element type; the output has it too or is float32")
     if not (k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
             and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
             and k_cache.shape[3] == head_dim):
@@ -633,7 +643,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _ptr(q), c_int64(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(out), c_int64(out.stride(0)),
         c_int(T), c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_int(k_cache.shape[2]),
-        c_float(scale), c_int(window), c_int(1 if sink else 0), c_int(_dt(q)), _stream()), "paged_attention")
+        c_float(scale), c_int(window), c_int(_attn_flags(sink, q, out)), c_int(_dt(q)), _stream()), "paged_attention")
     return out
 
 
@@ -734,8 +744,8 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
               "heads per kv head")
     if not (q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim)):
         _fail("q and the attention output must be [T, heads * head_dim]")
-    if not (q.dtype == k_cache.dtype == v_cache.dtype == out.dtype):
-        _fail("q, caches and output must share an element type")
+    if not _attn_types_ok(q, k_cache, v_cache, out):
+        _fail("q and caches must share an element type; the output has it too or is float32")
     if not (k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
             and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
             and k_cache.shape[3] == head_dim):
@@ -782,7 +792,7 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
             c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
             _ptr(out, 8), c_int64(out.stride(0)), c_int(n_tiles), c_int(T), c_int(num_heads), c_int(num_kv_heads),
-            c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(1 if sink else 0), c_int(n_splits), _ptr(cos),
+            c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(_attn_flags(sink, q, out)), c_int(n_splits), _ptr(cos),
             _ptr(sin), c_int(1 if fused_rope is not None else 0), _stream())
         if code == 3:
             _fail(f"split attention over the library's static scratch: {n_splits} splits x {T} tokens x {num_heads} "
@@ -794,8 +804,8 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
         _ptr(out, 8), c_int64(out.stride(0)), _ptr(part_o), _ptr(part_ml), c_int(n_tiles), c_int(T),
         c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale),
-        c_int(window), c_int(1 if sink else 0), c_int(n_splits), _ptr(cos), _ptr(sin), c_int(1 if fused_rope is not None else 0),
-        _stream()), "flash_attention")
+        c_int(window), c_int(_attn_flags(sink, q, out)), c_int(n_splits), _ptr(cos), _ptr(sin),
+        c_int(1 if fused_rope is not None else 0), _stream()), "flash_attention")
     return out
 
 
@@ -902,8 +912,8 @@ def flash_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
               "heads per kv head")
     if not (q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim)):
         _fail("q and the attention output must be [T, heads * head_dim]")
-    if not (q.dtype == k_cache.dtype == v_cache.dtype == out.dtype):
-        _fail("q, caches and output must share an element type")
+    if not _attn_types_ok(q, k_cache, v_cache, out):
+        _fail("q and caches must share an element type; the output has it too or is float32")
     if not (k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
             and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
             and k_cache.shape[3] == head_dim):
@@ -932,9 +942,9 @@ def flash_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
     _check(_lib().tl_flash_prefill(
         _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
-        _ptr(out, 8), c_int64(out.stride(0)), _ptr(part_o, 16), _ptr(part_ml), c_int(n_tiles), c_int(T),
+        _ptr(out, 16 if out.dtype == torch.float32 else 8), c_int64(out.stride(0)), _ptr(part_o, 16), _ptr(part_ml), c_int(n_tiles), c_int(T),
         c_int(num_heads), c_int(num_kv_heads),
-        c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(1 if sink else 0), c_int(tile_waves), c_int(n_splits),
+        c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(_attn_flags(sink, q, out)), c_int(tile_waves), c_int(n_splits),
         _stream()), "flash_prefill")
     return out
 
@@ -2212,7 +2222,8 @@ def attn_finish(a0: torch.Tensor, a1: Optional[torch.Tensor], gate: Optional[tor
                 gate_kind: Optional[str] = None, tail: int = 0) -> torch.Tensor:
     """Behind the attention kernel: of every head's D numbers the first vdim, o = a0 - lam * a1 (a1 None: o = a0),
     divided by the head's root mean square (`sub_norm`), times `scale`, times sigmoid(gate) (float32, one number per
-    token and head for "head", per element [T, heads * vdim] for "element"); z[t] = the heads side by side, then
+    token and head for "head", per element [T, heads * vdim] for "element"); a0 and a1 are float32 or of z's type;
+    z[t] = the heads side by side, then
     `tail` columns 1, 0, 0, ... (the one meets a bias kept as one more column of the next product's weight)."""
     _dev(a0, a1, gate, z)
     _rows_2d(a0, "attn_finish input")
@@ -2220,9 +2231,9 @@ def attn_finish(a0: torch.Tensor, a1: Optional[torch.Tensor], gate: Optional[tor
     T = a0.shape[0]
     _need(a0.shape[1] % heads == 0, "attn_finish: the input is [T, heads * D]")
     D = a0.shape[1] // heads
-    _need(0 < vdim <= D and vdim <= ATTN_PREPARE_MAX_DIM and z.dtype == a0.dtype and z.shape[0] == T
-          and z.shape[1] == heads * vdim + tail and 0 <= tail <= 64, "attn_finish: z is [T, heads * vdim + tail] of "
-          "the input's type")
+    _need(0 < vdim <= D and vdim <= ATTN_PREPARE_MAX_DIM and a0.dtype in (z.dtype, torch.float32) and z.shape[0] == T
+          and z.shape[1] == heads * vdim + tail and 0 <= tail <= 64, "attn_finish: z is [T, heads * vdim + tail]; the "
+          "input has its type or is float32")
     if a1 is not None:
         _need(a1.dtype == a0.dtype and a1.shape == a0.shape and a1.stride() == a0.stride(),
               "attn_finish: the second map has the first one's layout")
@@ -2235,8 +2246,8 @@ def attn_finish(a0: torch.Tensor, a1: Optional[torch.Tensor], gate: Optional[tor
     _check(_lib().tl_attn_finish(_ptr(a0), _ptr(a1), c_int64(a0.stride(0)), _ptr(gate if gate_kind else None),
                                  c_int64(gate.stride(0) if gate_kind else 0), _ptr(z), c_int64(z.stride(0)), c_int(T),
                                  c_int(heads), c_int(vdim), c_int(D), c_float(lam), c_int(1 if sub_norm else 0),
-                                 c_float(eps), c_float(scale), c_int(ATTN_GATES[gate_kind]), c_int(tail), c_int(_dt(z)),
-                                 _stream()), "attn_finish")
+                                 c_float(eps), c_float(scale), c_int(ATTN_GATES[gate_kind]), c_int(tail), c_int(_dt(a0)),
+                                 c_int(_dt(z)), _stream()), "attn_finish")
     return z
 
 

@@ -409,7 +409,8 @@ class GatedAttention(Attention):
                          self.eps, self.q_temp)
         outs = []
         for m in range(self.maps):
-            attn = ops.scratch("attention_out" if m == 0 else "attention_out2", (T, self.q_size), self.dtype, dev)
+            # float32 whatever the engine's type: the maps' difference, the head's norm and the gates follow in float32
+            attn = ops.scratch("attention_out" if m == 0 else "attention_out2", (T, self.q_size), torch.float32, dev)
             view = LayerCache({"k": k_caches[m], "v": cache.tensors["v"]}, cache.group, cache.write)
             outs.append(self._attend(q[m], ctx, view, attn))
         z = ops.scratch("attention_gated", (T, self.out_cols + self.out_tail), self.dtype, dev)
