@@ -13,7 +13,7 @@ Llama-3-8B shape; 64 requests of 1,024 tokens that nearly fill the cache at the 
 `--only` picks a part (for profiling), or one of the measurements that are not part of the line:
 `attention` (the attention kernels alone at contexts up to 131,072 tokens), `long_context` (the Llama-3-8B
 shape with 8 requests of 32,000 tokens and one of 131,000), `decode_shapes` (decode steps at the two larger
-shapes by batch), `host` (a step's wall time against its time on the GPU), `gesutar` and `fofapel` (those designs, as `lufazen`), `lufazen` (the Lufazen design,
+shapes by batch), `host` (a step's wall time against its time on the GPU), `vevapel`, `gesutar` and `fofapel` (those designs, as `lufazen`), `lufazen` (the Lufazen design,
 recurrent and latent-attention layers, at two sizes beside a Llama of equal size: prefill, decode, time by kernel).
 """
 import argparse
@@ -850,7 +850,62 @@ def gesutar_figures(args):
     return design_beside_llama(args, "gesutar", gesutar_config, bounds)
 
 
-def design_beside_llama(args, design, config_of, bounds_of):
+def vevapel_config(layers, width, ff, heads, vocab=32000, chunk=512):
+    """`layers` layer RUNS: layers - 2 layers in the order attention, delta, attention_2, of which the second and third
+    run twice (a loop over two layers).  Attention: heads of 128 keys and 128 values, four query heads a kv head, a query
+    temperature; delta: `heads` heads of 128 key channels and 128 values with q/k heads of their own, four taps;
+    attention_2: two score maps a head of 128 dims each (rotated on 64) over values of 128, chunks of 512 positions;
+    every layer with 16 routed experts of ff / 8, four a token (half of a dense layer's hidden units a token)."""
+    out = []
+    kv = max(1, heads // 4)
+    mlp = {"kind": "moe", "router": {"experts": 16, "top": 4}, "expert": {"ff": ff // 8}}
+    for i in range(max(3, layers - 2)):
+        if i % 3 == 0:
+            out.append({"type": "attention", "mlp": mlp,
+                        "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                  "q_temp": {"coef": 0.1, "every": 256}}})
+        elif i % 3 == 1:
+            out.append({"type": "delta", "mlp": mlp,
+                        "mixer": {"heads": heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4}})
+        else:
+            out.append({"type": "attention_2", "mlp": mlp,
+                        "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "diff": 0.3,
+                                  "mask": {"size": chunk}, "rot": {"base": 10000.0, "dims": 64}}})
+    return {"architecture": "Vevapel", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+            "embedding": {"scale": 1.0}, "layers": out, "loop": {"start": 1, "stop": 3, "times": 2}, "max_position": 8192}
+
+
+def vevapel_figures(args):
+    """The Vevapel design at two sizes beside the closest design of the tree, Lufazen (recurrent delta-rule layers among
+    attention layers, listed layer by layer), and a Llama, each of equal layer runs, width, feed-forward size, heads of
+    128 and vocabulary, as `lufazen_figures`; bounds for the kernels that this design runs."""
+    def bounds(dtype, heads, width, ff):
+        e = ELT[dtype]
+        T, ctx, B, chunk = PREFILL_TOKENS, PROMPT_LEN, 8, 512
+        kv = max(1, heads // 4)
+        return {
+            "attention prefill (flops of scores and values, causal)":
+                round(2.0 * heads * (T * T / 2) * 2 * 128 / (PEAK_TFLOPS[dtype] * 1e12) * 1e6, 1),
+            "attention decode b8 (the cached keys and values once)":
+                round(B * ctx * 2 * kv * 128 * e / (HBM_GBS * 1e9) * 1e6, 2),
+            "attention_2 prefill (flops of two maps' scores and values inside the chunks)":
+                round(2 * 2.0 * heads * T * (chunk / 2) * 2 * 128 / (PEAK_TFLOPS[dtype] * 1e12) * 1e6, 1),
+            "attention_2 decode b8 (two maps' cached keys and the values of a chunk once)":
+                round(B * min(ctx, chunk) * 3 * kv * 128 * e / (HBM_GBS * 1e9) * 1e6, 2),
+            "delta decode b8 (the states read and written)":
+                round(2.0 * B * heads * 128 * 128 * 4 / (HBM_GBS * 1e9) * 1e6, 2),
+            "delta_recurrence prefill (6 flops per state element and token, float32 vector units at 157 TFLOP/s)":
+                round(6.0 * T * heads * 128 * 128 / (157.3e12) * 1e6, 1),
+            "experts decode b8 (the weights of all 16 experts once)":
+                round(16 * 3 * width * (ff // 8) * e / (HBM_GBS * 1e9) * 1e6, 2),
+            "experts prefill (flops of four experts a token)":
+                round(2.0 * T * 4 * 3 * width * (ff // 8) / (PEAK_TFLOPS[dtype] * 1e12) * 1e6, 1),
+        }
+    return design_beside_llama(args, "vevapel", vevapel_config, bounds, beside=(("lufazen", lufazen_config),))
+
+
+def design_beside_llama(args, design, config_of, bounds_of, beside=()):
+    """`beside`: (name, config function) of further designs of the tree to measure at the same sizes."""
     import torch
     dtype = args.dtype
     out = {}
@@ -859,6 +914,7 @@ def design_beside_llama(args, design, config_of, bounds_of):
             layers = args.layers
         row = {"layers": layers, "width": width, "ff": ff, "heads": heads}
         for which, cfg in ((design, config_of(layers, width, ff, heads)),
+                           *((n, f(layers, width, ff, heads)) for n, f in beside),
                            ("llama", llama(layers, width, heads, heads, ff, 32000, 10000.0, 8192))):
             b = Bench(cfg, dtype, max_batch=8, total_new=args.steps + args.warmup + 200, block_size=args.block_size)
             r = {}
@@ -906,6 +962,9 @@ def run(args):
         return
     if args.only == "gesutar":
         print(json.dumps({"gesutar_beside_llama": gesutar_figures(args)}), flush=True)
+        return
+    if args.only == "vevapel":
+        print(json.dumps({"vevapel_beside_lufazen_and_llama": vevapel_figures(args)}), flush=True)
         return
     if args.only == "attention":
         print(json.dumps({"decode_attention": attention_sweep()}), flush=True)
@@ -982,7 +1041,7 @@ def main():
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--only", default="all",
                     choices=["all", "headline", "decode", "prefill", "fp32", "kernels", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host",
-                             "attention", "long_context", "decode_shapes", "lufazen", "fofapel", "gesutar"],
+                             "attention", "long_context", "decode_shapes", "lufazen", "fofapel", "gesutar", "vevapel"],
                     help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
                          "one of them (profiling); fp32: the float32 figures as the headline; kernels: decode with the time of "
                          "a step by kernel (torch's profiler); peaks / llama3_8b / "
@@ -990,7 +1049,8 @@ def main():
                          "attention kernels alone at contexts up to 131,072 tokens; long_context: the Llama-3-8B shape with "
                          "8 requests of 32,000 tokens and one of 131,000; decode_shapes: decode steps at the two larger shapes by batch; "
                          "lufazen: prefill and decode of the Lufazen design at two sizes beside a Llama of equal size, by kernel; "
-                         "fofapel, gesutar: the same for the Fofapel and the Gesutar design")
+                         "fofapel, gesutar: the same for the Fofapel and the Gesutar design; "
+                         "vevapel: the Vevapel design beside Lufazen and a Llama of equal size")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         if int(os.environ.get("RANK", "0")) == 0:

@@ -75,9 +75,11 @@ __global__ __launch_bounds__(kThreads) void layer_norm_kernel(const float* __res
 }
 
 // x[row] <- x[row] + mult * (LN(y[row]) * w + b); then, if w2 is given, out[row] = LN(x[row]) * w2 + b2 in TO: the
-// norm of whatever reads the stream next, formed while the row is in registers.  One workgroup a row; rows of up
-// to KEEP * kThreads elements.
-template <typename TO, int KEEP>
+// norm of whatever reads the stream next, formed while the row is in registers.  One workgroup a row.  Everything
+// the row needs (y, x, both norms' weights and biases) is requested before the first sum is taken, so the four sums
+// over the workgroup are all that stands between the loads and the stores.  VEC 4: rows of a multiple of four
+// elements, KEEP vectors of four a thread; VEC 1: any row, KEEP elements a thread.
+template <typename TO, int KEEP, int VEC>
 __global__ __launch_bounds__(kThreads) void layer_norm_add_kernel(const float* __restrict__ y, const float* __restrict__ w,
                                                                   const float* __restrict__ b, float* __restrict__ x,
                                                                   const float* __restrict__ w2, const float* __restrict__ b2,
@@ -88,50 +90,85 @@ __global__ __launch_bounds__(kThreads) void layer_norm_add_kernel(const float* _
   float* xr = x + row * hidden;
   const float* yr = y + row * hidden;
   const float inv_n = 1.f / (float)hidden;
-  float v[KEEP];
-  float s = 0.f;
+  constexpr int N = KEEP * VEC;
+  float v[N], xv[N], wv[N], bv[N], w2v[N], b2v[N];
 #pragma unroll
   for (int i = 0; i < KEEP; ++i) {
-    const int j = threadIdx.x + i * kThreads;
-    v[i] = j < hidden ? yr[j] : 0.f;
-    s += v[i];
+    const int j = (threadIdx.x + i * kThreads) * VEC;
+    const bool in = j < hidden;
+    if constexpr (VEC == 4) {
+      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      const f32x4 a = in ? *(const f32x4*)(yr + j) : z, c = in ? *(const f32x4*)(xr + j) : z;
+      const f32x4 d = in ? *(const f32x4*)(w + j) : z, e = in ? *(const f32x4*)(b + j) : z;
+      const f32x4 f = (in && w2) ? *(const f32x4*)(w2 + j) : z, g = (in && w2) ? *(const f32x4*)(b2 + j) : z;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        v[i * 4 + u] = a[u];
+        xv[i * 4 + u] = c[u];
+        wv[i * 4 + u] = d[u];
+        bv[i * 4 + u] = e[u];
+        w2v[i * 4 + u] = f[u];
+        b2v[i * 4 + u] = g[u];
+      }
+    } else {
+      v[i] = in ? yr[j] : 0.f;
+      xv[i] = in ? xr[j] : 0.f;
+      wv[i] = in ? w[j] : 0.f;
+      bv[i] = in ? b[j] : 0.f;
+      w2v[i] = (in && w2) ? w2[j] : 0.f;
+      b2v[i] = (in && w2) ? b2[j] : 0.f;
+    }
   }
+  auto inside = [&](int i) { return (threadIdx.x + (i / VEC) * kThreads) * VEC + i % VEC < hidden; };
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < N; ++i) s += v[i];
   float mean = block_sum<kWaves>(s, red) * inv_n;
   float q = 0.f;
 #pragma unroll
-  for (int i = 0; i < KEEP; ++i) {
-    const int j = threadIdx.x + i * kThreads;
-    const float d = j < hidden ? v[i] - mean : 0.f;
+  for (int i = 0; i < N; ++i) {
+    const float d = inside(i) ? v[i] - mean : 0.f;
     q += d * d;
   }
   float r = 1.f / sqrtf(block_sum<kWaves>(q, red) * inv_n + eps);
   s = 0.f;
 #pragma unroll
-  for (int i = 0; i < KEEP; ++i) {
-    const int j = threadIdx.x + i * kThreads;
-    if (j < hidden) {
-      v[i] = fmaf(mult, (v[i] - mean) * r * w[j] + b[j], xr[j]);
-      xr[j] = v[i];
-    } else {
-      v[i] = 0.f;
-    }
+  for (int i = 0; i < N; ++i) {
+    v[i] = inside(i) ? fmaf(mult, (v[i] - mean) * r * wv[i] + bv[i], xv[i]) : 0.f;
     s += v[i];
+  }
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int j = (threadIdx.x + i * kThreads) * VEC;
+    if (j < hidden) {
+      if constexpr (VEC == 4) *(f32x4*)(xr + j) = f32x4{v[i * 4], v[i * 4 + 1], v[i * 4 + 2], v[i * 4 + 3]};
+      else xr[j] = v[i];
+    }
   }
   if (!w2) return;
   mean = block_sum<kWaves>(s, red) * inv_n;
   q = 0.f;
 #pragma unroll
-  for (int i = 0; i < KEEP; ++i) {
-    const int j = threadIdx.x + i * kThreads;
-    const float d = j < hidden ? v[i] - mean : 0.f;
+  for (int i = 0; i < N; ++i) {
+    const float d = inside(i) ? v[i] - mean : 0.f;
     q += d * d;
   }
   r = 1.f / sqrtf(block_sum<kWaves>(q, red) * inv_n + eps2);
   TO* dst = out + row * hidden;
 #pragma unroll
   for (int i = 0; i < KEEP; ++i) {
-    const int j = threadIdx.x + i * kThreads;
-    if (j < hidden) dst[j] = from_f32<TO>((v[i] - mean) * r * w2[j] + b2[j]);
+    const int j = (threadIdx.x + i * kThreads) * VEC;
+    if (j < hidden) {
+      if constexpr (VEC == 4) {
+        typedef __attribute__((ext_vector_type(4))) decltype(from_f32<TO>(0.f)) out4;
+        out4 o;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) o[u] = from_f32<TO>((v[i * 4 + u] - mean) * r * w2v[i * 4 + u] + b2v[i * 4 + u]);
+        *(out4*)(dst + j) = o;
+      } else {
+        dst[j] = from_f32<TO>((v[i] - mean) * r * w2v[i] + b2v[i]);
+      }
+    }
   }
 }
 
@@ -139,10 +176,22 @@ template <typename TO>
 int launch_add(const float* y, const float* w, const float* b, float* x, const float* w2, const float* b2, TO* out, int n,
                int hidden, float mult, float eps, float eps2, hipStream_t stream) {
   dim3 g(n), blk(kThreads);
-  if (hidden <= 8 * kThreads)
-    hipLaunchKernelGGL((layer_norm_add_kernel<TO, 8>), g, blk, 0, stream, y, w, b, x, w2, b2, out, hidden, mult, eps, eps2);
-  else
-    hipLaunchKernelGGL((layer_norm_add_kernel<TO, 32>), g, blk, 0, stream, y, w, b, x, w2, b2, out, hidden, mult, eps, eps2);
+#define TL_LNA(KEEP, VEC)                                                                                            \
+  hipLaunchKernelGGL((layer_norm_add_kernel<TO, KEEP, VEC>), g, blk, 0, stream, y, w, b, x, w2, b2, out, hidden, mult, \
+                     eps, eps2)
+  const uintptr_t ptrs = (uintptr_t)y | (uintptr_t)w | (uintptr_t)b | (uintptr_t)x | (uintptr_t)w2 | (uintptr_t)b2 | (uintptr_t)out;
+  if (hidden % 4 == 0 && (ptrs & 15) == 0) {      // vectors of four need 16-byte boundaries
+    const int vecs = hidden / 4;
+    if (vecs <= kThreads) TL_LNA(1, 4);
+    else if (vecs <= 2 * kThreads) TL_LNA(2, 4);
+    else if (vecs <= 4 * kThreads) TL_LNA(4, 4);
+    else TL_LNA(8, 4);
+  } else {
+    if (hidden <= 4 * kThreads) TL_LNA(4, 1);
+    else if (hidden <= 16 * kThreads) TL_LNA(16, 1);
+    else TL_LNA(32, 1);
+  }
+#undef TL_LNA
   return tl_launch_status();
 }
 

@@ -115,7 +115,7 @@ __device__ __forceinline__ int expert_of(const int32_t* tokens, const int32_t* t
 }
 
 // What follows an expert's first product: nothing, or the square of max(., 0).
-constexpr int kActNone = 0, kActRelu2 = 1;
+constexpr int kActNone = 0, kActRelu2 = 1, kActSiluGate = 2;     // the last one in the per-row first product only
 __device__ __forceinline__ float activate(float v, int act) {
   if (act == kActRelu2) {
     v = fmaxf(v, 0.f);
@@ -124,7 +124,9 @@ __device__ __forceinline__ float activate(float v, int act) {
   return v;
 }
 
-// out[t * top + j, n] = act(sum_k a[t, k] * w[e(t, j)][n, k])
+// out[t * top + j, n] = act(sum_k a[t, k] * w[e(t, j)][n, k]); with the gated activation an expert's N rows are
+// [gate rows | up rows] and out[t * top + j, n] = silu(gate_n) * up_n for n < N / 2, formed from the float32 sums
+// (a wave's four dot products are then two gates and their two ups).
 template <typename T>
 __global__ __launch_bounds__(kThreads) void table_moe_up_kernel(const T* __restrict__ a, int64_t a_stride,
                                                                 const T* __restrict__ w,
@@ -138,6 +140,21 @@ __global__ __launch_bounds__(kThreads) void table_moe_up_kernel(const T* __restr
   const T* arow = a + (int64_t)t * a_stride;
   const T* we = w + (int64_t)e * N * K;
   const int n0 = blockIdx.y * kCols + wave * (kCols / kWaves);
+  if (act == kActSiluGate) {
+    const int F = N / 2;
+    for (int n = n0; n < min(F, n0 + kCols / kWaves); n += 2) {
+      const T* wr[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) wr[c] = we + (int64_t)((c / 2) * F + min(n + (c & 1), F - 1)) * K;
+      float v[4];
+      dot_lanes4(arow, wr, K, lane, v);
+      if (lane < 2 && n + lane < F) {
+        const float g = v[lane], u = v[lane + 2];
+        out[(int64_t)row * F + n + lane] = from_f32<T>(g / (1.f + expf(-g)) * u);
+      }
+    }
+    return;
+  }
   for (int n = n0; n < min(N, n0 + kCols / kWaves); n += 4) {
     const T* wr[4];
 #pragma unroll
@@ -588,11 +605,12 @@ int tl_table_moe_up(const void* a, int64_t a_stride, const void* w, const int32_
                     int n_tokens, int top, int experts, int vocab, int N, int K, int act, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (top <= 0 || experts <= 0 || vocab <= 0 || N <= 0 || K <= 0 || a_stride < K || !a || !w || !table || !out ||
-      (act != kActNone && act != kActRelu2) || (!tokens && vocab < n_tokens) ||
-      (int64_t)n_tokens * top > 0x7fffffff || (N + kColsFew - 1) / kColsFew > 65535)
+      (act != kActNone && act != kActRelu2 && act != kActSiluGate) || (act == kActSiluGate && (N & 1)) ||
+      (!tokens && vocab < n_tokens) || (int64_t)n_tokens * top > 0x7fffffff || (N + kColsFew - 1) / kColsFew > 65535)
     return TL_ERR_ARG;
   const int kCols = (int64_t)n_tokens * top <= kFewRows ? kColsFew : kColsWide;
-  dim3 g(n_tokens * top, (N + kCols - 1) / kCols), b(kThreads);
+  const int n_out = act == kActSiluGate ? N / 2 : N;      // output columns
+  dim3 g(n_tokens * top, (n_out + kCols - 1) / kCols), b(kThreads);
   if (dtype == 0)
     hipLaunchKernelGGL(table_moe_up_kernel<float>, g, b, 0, stream, (const float*)a, a_stride, (const float*)w, tokens,
                        table, (float*)out, top, experts, vocab, N, K, act, kCols);

@@ -100,8 +100,9 @@ __global__ void head_gate_kernel(const T* __restrict__ a, int64_t a_stride, cons
   z[t * z_stride + c] = from_f32<T>(to_f32(a[t * a_stride + c]) * gate * scale);
 }
 
-// The general form of the step between the product that reads the mixer's input and the attention kernel: one
-// workgroup a token, a wave a unit.  Row t of p (float32) holds q as `q_units` units of `dim` numbers, then k as
+// The general form of the step between the product that reads the mixer's input and the attention kernel: the
+// workgroups (t, 0 .. gridDim.y - 1) share a token's units and values out, a wave a unit at a time (steps of few
+// tokens get many workgroups a token; each forms the sums of the whole-projection norm for itself).  Row t of p (float32) holds q as `q_units` units of `dim` numbers, then k as
 // `k_units` units, then v as `nkv` heads of `vdim` numbers (from column v_off); a unit is one score map of one
 // head, unit u = head * maps + map.  In this order, each step an option:
 //   a = p + bias                                      (bias over [q | k | v], or null)
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(kPrepThreads) void attn_prepare_kernel(
   const float* cs = rot ? cos_t + (int64_t)pos * half : nullptr;
   const float* sn = rot ? sin_t + (int64_t)pos * half : nullptr;
   const int64_t page_row = slot >= 0 ? (int64_t)(slot / block_size) * nkv * block_size + slot % block_size : 0;
-  for (int u = wave; u < q_units + k_units; u += kPrepWaves) {
+  for (int u = blockIdx.y * kPrepWaves + wave; u < q_units + k_units; u += gridDim.y * kPrepWaves) {
     const bool is_key = u >= q_units;
     if (is_key && slot < 0) continue;
     const int uu = is_key ? u - q_units : u;
@@ -202,7 +203,7 @@ __global__ __launch_bounds__(kPrepThreads) void attn_prepare_kernel(
     }
   }
   if (slot < 0) return;
-  for (int c = tid; c < nkv * D; c += kPrepThreads) {
+  for (int c = blockIdx.y * kPrepThreads + tid; c < nkv * D; c += gridDim.y * kPrepThreads) {
     const int g = c / D, d = c - g * D;
     float a = 0.f;
     if (d < vdim) {
@@ -324,7 +325,10 @@ int tl_attn_prepare(const float* p, int64_t p_stride, const float* bias, const f
   if (whole_norm && !norm_w) return TL_ERR_ARG;
   if (slot_mapping && (!k_cache0 || !v_cache || (maps == 2 && !k_cache1))) return TL_ERR_ARG;
   if (interleaved != 0 && interleaved != 1) return TL_ERR_ARG;
-  dim3 g(n_tokens), b(kPrepThreads);
+  // about 256 workgroups in all where the units allow it, a wave with at least one unit
+  const int units = (heads + nkv) * maps, most = (units + kPrepWaves - 1) / kPrepWaves;
+  const int share = n_tokens >= 256 ? 1 : (256 / n_tokens < most ? 256 / n_tokens : most);
+  dim3 g(n_tokens, share), b(kPrepThreads);
   if (dtype == 0)
     hipLaunchKernelGGL(attn_prepare_kernel<float>, g, b, 0, stream, p, p_stride, bias, norm_w, positions, cos_t, sin_t,
                        slot_mapping, (float*)q_out, q_stride, q_map_stride, (float*)k_cache0, (float*)k_cache1,

@@ -1840,21 +1840,25 @@ def tanh_rows(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 
 # ------------------------------------------------------------ experts looked up in a table
 MOE_ACTIVATIONS = {None: 0, "relu2": 1}      # what may follow an expert's first product (csrc/moe.hip)
+MOE_GATED = "swiglu"                         # `table_moe_up` only: an expert's rows are [gate | up], out = silu(gate) * up
 
 
 def table_moe_up(a: torch.Tensor, w: torch.Tensor, tokens: Optional[torch.Tensor], table: torch.Tensor, out: torch.Tensor,
                  act: Optional[str] = None) -> torch.Tensor:
     """out[t * top + j] = act(w[table[tokens[t], j]] @ a[t]); a [T, K], w [E, N, K] of one type, table int32 [vocab, top],
     out contiguous [T * top, N].  tokens None: the table has a row per row of a (the experts a router chose).
-    act None or "relu2" (the square of max(., 0))."""
+    act None, "relu2" (the square of max(., 0)) or "swiglu": an expert's N rows are [gate rows | up rows] and out
+    [T * top, N / 2] = silu(gate) * up, formed from the float32 sums."""
     _dev(a, w, tokens, table, out)
-    _need(act in MOE_ACTIVATIONS, f"table_moe_up: activation {act!r} is not built")
+    _need(act in MOE_ACTIVATIONS or act == MOE_GATED, f"table_moe_up: activation {act!r} is not built")
     _rows_2d(a, "table_moe_up input")
     T, K = a.shape
     E, N, _ = w.shape
     V, top = table.shape
     _need(w.is_contiguous() and w.shape[2] == K and w.dtype == a.dtype == out.dtype, "table_moe_up: w is contiguous [E, N, K]")
-    _need(out.is_contiguous() and tuple(out.shape) == (T * top, N), "table_moe_up: the output is contiguous [T * top, N]")
+    n_out = N // 2 if act == MOE_GATED else N
+    _need(N % 2 == 0 or act != MOE_GATED, "table_moe_up: gated experts have an even number of rows")
+    _need(out.is_contiguous() and tuple(out.shape) == (T * top, n_out), f"table_moe_up: the output is contiguous [T * top, {n_out}]")
     _i32(table)
     if tokens is not None:
         _i32(tokens)
@@ -1862,8 +1866,9 @@ def table_moe_up(a: torch.Tensor, w: torch.Tensor, tokens: Optional[torch.Tensor
     else:
         _need(V >= T and table.is_contiguous(), "table_moe_up: without token ids the table has a row per row of the input")
     _check(_lib().tl_table_moe_up(_ptr(a), c_int64(a.stride(0)), _ptr(w), _ptr(tokens), _ptr(table), _ptr(out), c_int(T),
-                                  c_int(top), c_int(E), c_int(V), c_int(N), c_int(K), c_int(MOE_ACTIVATIONS[act]),
-                                  c_int(_dt(a)), _stream()), "table_moe_up")
+                                  c_int(top), c_int(E), c_int(V), c_int(N), c_int(K),
+                                  c_int(2 if act == MOE_GATED else MOE_ACTIVATIONS[act]), c_int(_dt(a)), _stream()),
+           "table_moe_up")
     return out
 
 

@@ -274,12 +274,7 @@ class RoutedMoE(FeedForward):
             # few rows (decoding) and float32: each row against its own expert's weights, the activation in
             # the first product's kernel
             z = ops.scratch("moe_gated", (rows, F), self.dtype, dev)
-            if self.gated:
-                gup = ops.scratch("moe_gate_up", (rows, 2 * F), self.dtype, dev)
-                ops.table_moe_up(h, self.w_up, None, ids, gup, None)
-                ops.silu_mul(gup, z)
-            else:
-                ops.table_moe_up(h, self.w_up, None, ids, z, self.activation)
+            ops.table_moe_up(h, self.w_up, None, ids, z, ops.MOE_GATED if self.gated else self.activation)
             ops.table_moe_down(z, self.w_down, None, ids, out, 1.0, base, None, wts)
         return out
 
