@@ -869,7 +869,7 @@ def vevapel_config(layers, width, ff, heads, vocab=32000, chunk=512):
                         "mixer": {"heads": heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4}})
         else:
             out.append({"type": "attention_2", "mlp": mlp,
-                        "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "diff": 0.3,
+                        "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "diff": 0.2,
                                   "mask": {"size": chunk}, "rot": {"base": 10000.0, "dims": 64}}})
     return {"architecture": "Vevapel", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
             "embedding": {"scale": 1.0}, "layers": out, "loop": {"start": 1, "stop": 3, "times": 2}, "max_position": 8192}

@@ -56,7 +56,7 @@ def causal(positions):
 
 
 def same_chunk(positions, size: int):
-    """Causal, and only inside the query's own run of `size` positions counted from position 0."""
+    """Causal, and only inside the query's own run of `size` positions (runs begin at multiples of `size`)."""
     i, j = positions[:, None], positions[None, :]
     return (j <= i) & (torch.div(i, size, rounding_mode="floor") == torch.div(j, size, rounding_mode="floor"))
 
@@ -127,7 +127,7 @@ def attention_2(h, w, m, eps, positions):
 
 # -------------------------------------------------------------- mixer: the delta rule
 def short_conv(x, taps_w):
-    """x [T, C], taps_w [C, taps]: y[t, c] = sum_j taps_w[c, j] x[t - (taps - 1) + j, c], zeros before the start."""
+    """x [T, C], taps_w [C, taps]: y[t, c] = sum_j taps_w[c, j] x[t - (taps - 1) + j, c], inputs ahead of the sequence count as zero."""
     T, taps = x.shape[0], taps_w.shape[1]
     pad = torch.cat([torch.zeros((taps - 1, x.shape[1]), dtype=x.dtype), x], dim=0)
     y = torch.zeros_like(x)

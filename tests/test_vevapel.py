@@ -21,13 +21,13 @@ def _decoder(cfg, dtype="float32"):
 
 def test_reader_takes_every_size_from_the_configuration():
     typed, spec, dec = _decoder(MIX_A)
-    assert (typed.vocab, typed.width, typed.norm_eps, typed.embedding_scale, typed.residual_mult) == (301, 64, 1e-5, 3.0, 0.7)
+    assert (typed.vocab, typed.width, typed.norm_eps, typed.embedding_scale, typed.residual_mult) == (301, 64, 1e-5, 2.5, 0.6)
     a = typed.layers[0].mixer
-    assert (a.heads, a.kv_heads, a.dim, a.vdim, a.temp_coef, a.temp_every, a.scale) == (4, 2, 24, 16, 0.5, 16, 2.0 * 24 ** -0.5)
+    assert (a.heads, a.kv_heads, a.dim, a.vdim, a.temp_coef, a.temp_every, a.scale) == (4, 2, 24, 16, 0.4, 16, 2.0 * 24 ** -0.5)
     d = typed.layers[1].mixer
     assert (d.heads, d.kv_heads, d.dim, d.vdim, d.conv) == (4, 2, 16, 8, 4)
     b = typed.layers[5].mixer
-    assert (b.heads, b.kv_heads, b.dim, b.vdim, b.diff, b.chunk, b.rot_dims, b.rot_base) == (2, 1, 32, 16, 0.6, 7, 32, 50000.0)
+    assert (b.heads, b.kv_heads, b.dim, b.vdim, b.diff, b.chunk, b.rot_dims, b.rot_base) == (2, 1, 32, 16, 0.6, 7, 32, 40000.0)
     m = typed.layers[0].mlp
     assert (m.experts, m.top, m.ff) == (6, 2, 24) and typed.layers[2].mlp is None
     assert (typed.loop.start, typed.loop.stop, typed.loop.times) == (1, 4, 3)
@@ -35,7 +35,7 @@ def test_reader_takes_every_size_from_the_configuration():
     assert tb.loop is None and tb.layers[2].mixer.temp_every == 0           # no temperature
     assert tb.layers[4].mixer.chunk == 0 and tb.layers[3].mixer.rot_dims == 0  # no mask, no rotation
     assert spec.architecture == "Vevapel"
-    assert dec.layers[0].block.mult == 0.7 and dec.embedding.scale == 3.0
+    assert dec.layers[0].block.mult == 0.6 and dec.embedding.scale == 2.5
 
 
 def test_plan_of_a_repeated_run():
@@ -151,7 +151,7 @@ def test_masks():
     assert ch[4].tolist() == [False] * 4 + [True] + [False] * 5                   # a chunk's first token sees itself
     assert ch[3].tolist() == [True] * 4 + [False] * 6
     assert plain.causal(pos)[3].tolist() == [True] * 4 + [False] * 6
-    # chunks are counted from position 0 whatever the first position given is
+    # a chunk begins at a multiple of its size whatever the first position given is
     assert plain.same_chunk(torch.arange(6, 9), 4)[2].tolist() == [False, False, True]
 
 

@@ -26,11 +26,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # compared in float32 and, with logits that are apart, at the part itself).  A fault of a mechanism (a key
 # off by one, a chunk's edge, a lost state, a pass's vector left out) moves a row by its whole size in
 # either precision.  The float32 figure: the plain model itself, run in float32, differs from its float64 run by
-# up to 3.3e-4 of a row on the liveliest model here (twelve layer runs, scores sharpened three times), by 8e-5 and
-# less on the others.  The bfloat16 models are also tamed in their residual multiplier (`vevapel_util.tame`):
+# up to 3.2e-4 of a row on the liveliest model here (twelve layer runs, scores sharpened three times; the engine, whose
+# sums run in other orders, by up to 5.3e-4), by 8e-5 and less on the others.  The bfloat16 models are also tamed in
+# their residual multiplier (`vevapel_util.tame`):
 # rounding nothing but every sublayer's input to bfloat16 in the plain model (`round_inputs`, the one rounding no
-# bfloat16 engine can avoid) then moves a row by 2e-2 at worst, where the untamed model moves by 1.8e-1.
-TOL = {"float32": 5e-4, "bfloat16": 1e-1}
+# bfloat16 engine can avoid) then moves a row by 1.7e-2 at worst, where the untamed model moves by 1.2e-1.
+TOL = {"float32": 1e-3, "bfloat16": 1e-1}
 LENGTHS = {"A": [70, 133, 33, 200, 97, 64], "B": [1, 9, 40, 100, 150, 57], "odd": [31, 2, 77, 50],
            "loop_all": [30, 3, 66], "loop_one": [45, 8, 90, 2], "attention": [40, 75, 130, 9], "diff": [40, 75, 130, 9],
            "delta": [24, 121, 48, 5], "moe": [24, 121, 48, 5]}
@@ -138,9 +139,8 @@ def test_odd_sizes_in_a_bfloat16_engine(tmp_path_factory):
     with pytest.warns(RuntimeWarning, match="served in float32"):
         runner = make_runner(folder, "bfloat16", block, max(peak, max(r64(len(t)) for t in reqs.values())))
     assert runner.decoder.dtype == torch.float32
-    # (the plain model itself, run in float32, differs from its float64 run by up to 1.4e-3 on this checkpoint)
     for st in (steps, traces.portions(reqs)):
-        check(replay(runner, st), st, ref, 2e-3)
+        check(replay(runner, st), st, ref, TOL["float32"])
         assert all_free(runner)
 
 
@@ -192,9 +192,9 @@ def test_layer_sizes_of_a_larger_model(dtype, tmp_path):
     second request."""
     from vevapel_util import attention, attention_2, delta, layer, model, moe
     big = model(256, 1031, [
-        layer(attention(16, 4, 128, 128, (0.5, 64), 128 ** -0.5), moe(16, 4, 64)),
+        layer(attention(16, 4, 128, 128, (0.3, 50), 128 ** -0.5), moe(16, 4, 64)),
         layer(delta(8, 4, 128, 128, 4), moe(12, 3, 32)),
-        layer(attention_2(8, 4, 64, 128, 200, 32, 0.3, 500000.0, 64 ** -0.5), moe(8, 2, 64)),
+        layer(attention_2(8, 4, 64, 128, 180, 32, 0.2, 500000.0, 64 ** -0.5), moe(8, 2, 64)),
     ], loop=(0, 3, 2), scale=8.0)
     cfg = tame(big) if dtype == "bfloat16" else big
     folder, w = make_folder(tmp_path, cfg, seed=5, store=torch.bfloat16 if dtype == "bfloat16" else torch.float32,
@@ -357,7 +357,7 @@ ATTENTION_KERNELS = ["general float32", "general bfloat16", "matrix cores float3
 
 
 @pytest.mark.parametrize("kernel", ATTENTION_KERNELS)
-@pytest.mark.parametrize("chunk", [40, 1, 17, 64, 200])
+@pytest.mark.parametrize("chunk", [40, 1, 17, 64, 150])
 def test_chunked_mask_finds_one_key(kernel, chunk):
     """One query per place of interest is aligned with one key (and scaled so that this score stands out): the result
     must be that key's value.  Keys at the chunk's first place, at both sides of page edges, the query's own position,

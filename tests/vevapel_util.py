@@ -12,7 +12,7 @@ import torch
 from fofapel_util import as_double, rounded, row_err  # noqa: F401  (the same comparisons serve every design)
 
 
-def attention(heads, kv_heads, dim, vdim, q_temp=(0.5, 16), scale=None):
+def attention(heads, kv_heads, dim, vdim, q_temp=(0.4, 16), scale=None):
     m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
          "scale": float(scale if scale is not None else 2.0 * dim ** -0.5)}
     if q_temp:
@@ -20,7 +20,7 @@ def attention(heads, kv_heads, dim, vdim, q_temp=(0.5, 16), scale=None):
     return {"type": "attention", "mixer": m}
 
 
-def attention_2(heads, kv_heads, dim, vdim, chunk, rot_dims, diff=0.3, base=10000.0, scale=None):
+def attention_2(heads, kv_heads, dim, vdim, chunk, rot_dims, diff=0.25, base=10000.0, scale=None):
     m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "diff": diff,
          "scale": float(scale if scale is not None else 2.0 * dim ** -0.5)}
     if chunk:
@@ -42,7 +42,7 @@ def layer(mixer, mlp):
     return dict(mixer, mlp=mlp)
 
 
-def model(width, vocab, layers, loop=None, mult=0.7, scale=3.0, eps=1e-5):
+def model(width, vocab, layers, loop=None, mult=0.6, scale=2.5, eps=1e-5):
     cfg = {"architecture": "Vevapel", "vocab": vocab, "width": width, "norm": {"eps": eps}, "residual_mult": mult,
            "embedding": {"scale": scale}, "layers": layers}
     if loop:
@@ -54,12 +54,12 @@ def model(width, vocab, layers, loop=None, mult=0.7, scale=3.0, eps=1e-5):
 # chunks of 24 and 7 positions and none, part and all of a map rotated, temperatures that step every 16 and every 5
 # positions, 2 to 4 taps, a layer without feed-forward; layers 1 to 3 run three times
 MIX_A = model(64, 301, [
-    layer(attention(4, 2, 24, 16, (0.5, 16)), moe(6, 2, 24)),
+    layer(attention(4, 2, 24, 16, (0.4, 16)), moe(6, 2, 24)),
     layer(delta(4, 2, 16, 8, 4), moe(4, 1, 16)),
-    layer(attention_2(4, 2, 16, 24, 24, 8, 0.3, 1000.0), None),
+    layer(attention_2(4, 2, 16, 24, 24, 8, 0.35, 1000.0), None),
     layer(attention(3, 3, 8, 40, (1.5, 5)), moe(8, 3, 8)),
     layer(delta(2, 2, 32, 16, 2), moe(3, 3, 16)),
-    layer(attention_2(2, 1, 32, 16, 7, 32, 0.6, 50000.0), moe(5, 2, 8)),
+    layer(attention_2(2, 1, 32, 16, 7, 32, 0.6, 40000.0), moe(5, 2, 8)),
 ], loop=(1, 4, 3))
 
 # no loop; one head, twenty heads (two tiles of heads), a chunk of one position (a token sees itself alone), a chunk
@@ -77,7 +77,7 @@ MIX_B = model(128, 257, [
 LOOP_ALL = model(64, 199, [layer(attention(2, 1, 16, 16, (0.3, 7)), moe(4, 2, 16)), layer(delta(2, 1, 16, 16, 4), None)],
                  loop=(0, 2, 1))
 LOOP_ONE = model(64, 199, [layer(delta(2, 2, 16, 8, 4), moe(3, 1, 8)), layer(attention_2(2, 2, 16, 16, 10, 16), moe(4, 2, 16)),
-                           layer(attention(4, 1, 16, 8, (0.5, 9)), None)], loop=(1, 2, 5), mult=0.4)
+                           layer(attention(4, 1, 16, 8, (0.6, 9)), None)], loop=(1, 2, 5), mult=0.4)
 
 # sizes that are multiples of nothing (float32 only)
 ODD = model(50, 199, [
@@ -86,7 +86,7 @@ ODD = model(50, 199, [
     layer(attention_2(2, 2, 6, 11, 13, 4, 0.25, 777.0), moe(2, 1, 7)),
 ], loop=(0, 2, 2), scale=0.5)
 
-ONLY_ATTENTION = model(64, 199, [layer(attention(6, 2, 16, 8, (0.5, 8)), None)])
+ONLY_ATTENTION = model(64, 199, [layer(attention(6, 2, 16, 8, (0.8, 8)), None)])
 ONLY_DIFF = model(64, 199, [layer(attention_2(4, 2, 16, 24, 20, 8), None)])
 ONLY_DELTA = model(64, 199, [layer(delta(4, 2, 16, 24, 4), None)])
 ONLY_MOE = model(64, 199, [layer(attention(2, 2, 8, 8, None), moe(8, 3, 16))])
@@ -108,9 +108,9 @@ def every_expert(cfg):
 def tame(cfg, mult=0.3):
     """The model a bfloat16 engine is compared on: every expert chosen by every token, and a sublayer's normed result
     added times at most `mult`.  A norm sits behind every sublayer, so a sublayer's relative rounding error reaches
-    the stream undamped, times the multiplier; at 0.7 and more, twelve layer runs double it from run to run (rounding
-    nothing but the sublayers' inputs to bfloat16 moves a row of the plain model by up to 1.8e-1), at 0.3 they do not
-    (2e-2)."""
+    the stream undamped, times the multiplier; at 0.6 and more, twelve layer runs nearly double it from run to run
+    (rounding nothing but the sublayers' inputs to bfloat16 moves a row of the plain model by up to 1.2e-1), at 0.3 they
+    do not (1.7e-2)."""
     out = every_expert(cfg)
     out["residual_mult"] = min(out.get("residual_mult", 1.0), mult)
     return out
@@ -130,10 +130,10 @@ def random_config(seed, multiple=8):
         dim, vdim = m * rng.randrange(1, 9), m * rng.randrange(1, 9)
         kind = rng.choice(["attention", "attention_2", "delta"])
         if kind == "attention":
-            mix = attention(heads, kv, dim, vdim, rng.choice([None, (0.5, 64), (1.0, 3), (0.2, 1)]))
+            mix = attention(heads, kv, dim, vdim, rng.choice([None, (0.4, 32), (1.0, 3), (0.2, 1)]))
         elif kind == "attention_2":
             mix = attention_2(heads, kv, dim, vdim, rng.choice([0, 1, 2, 5, 16, 31, 64, 100, 5000]),
-                              rng.choice([0, dim, max(2, dim // 2 // 2 * 2)]), rng.choice([0.1, 0.3, 0.8]),
+                              rng.choice([0, dim, max(2, dim // 2 // 2 * 2)]), rng.choice([0.1, 0.35, 0.8]),
                               rng.choice([100.0, 10000.0, 250000.0]))
         else:
             mix = delta(heads, kv, dim, vdim, rng.choice([2, 3, 4]))
@@ -146,7 +146,7 @@ def random_config(seed, multiple=8):
     if rng.random() < 0.7:
         start = rng.randrange(0, len(layers))
         loop = (start, rng.randrange(start + 1, len(layers) + 1), rng.randrange(1, 4))
-    return model(width, rng.randrange(90, 700), layers, loop, mult=rng.choice([1.0, 0.7, 0.3]),
+    return model(width, rng.randrange(90, 700), layers, loop, mult=rng.choice([1.0, 0.6, 0.3]),
                  scale=rng.choice([1.0, 4.0, 11.0]), eps=rng.choice([1e-5, 1e-6, 1e-4]))
 
 

@@ -2,8 +2,8 @@
 
 config.json of this design is nested: `embedding.scale`; `layers` (the layers in order, each with `type`, which
 mixer: `attention`, `delta` or `attention_2`; `mixer`, its sizes and constants; and `mlp`, a mixture of experts or
-null for none); `loop` (`start`, `stop`, `times`: layers start .. stop - 1 run `times` times in a row with the same
-weights; absent: every layer runs once); `norm.eps`; `residual_mult`; `vocab`; `width`.  Every size and constant
+null for none); `loop` (`start`, `stop`, `times`: the layers from `start` up to but not including `stop` are run `times` times over on
+the same weights, pass after pass; absent: every layer runs once); `norm.eps`; `residual_mult`; `vocab`; `width`.  Every size and constant
 that can differ between models of the design comes from there; a layer has its own.
 """
 from __future__ import annotations

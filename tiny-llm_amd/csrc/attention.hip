@@ -22,8 +22,8 @@
 namespace {
 
 // The first key position a row at position `pos` sees (it sees up to its own): with window > 0 the last
-// `window` positions; with window < 0 its own run of -window positions, runs counted from position 0 of
-// the sequence (a chunked mask); with 0 everything.  Never decreases as pos grows.
+// `window` positions; with window < 0 its own run of -window positions, runs beginning at multiples of -window
+// (a chunked mask); with 0 everything.  Never decreases as pos grows.
 __device__ __forceinline__ int first_visible_key(int pos, int window) {
   if (window > 0) return pos + 1 > window ? pos + 1 - window : 0;
   if (window < 0 && pos > 0) return pos / (-window) * (-window);

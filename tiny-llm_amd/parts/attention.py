@@ -267,7 +267,7 @@ class GatedAttention(Attention):
         q times 1 + coef ln(floor((pos + 1) / every) + 1)                              `q_temp=(coef, every)`
         keys seen: all earlier ones, the last `window`, or those of the row's own run of `chunk` positions
         `maps=2`: two score maps per head (q and k hold [map 1 | map 2] head by head) over the same values,
-                  o = a1 - lambda a2, lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff (one number for the layer)
+                  o = a1 - lambda a2, lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff (a scalar of the layer)
         o divided by its root mean square over the head, no weight (`sub_norm`), times `out_scale`
         o times sigmoid(W_g h): one number per head (`gate="head"`) or per element (`gate="element"`)
 
@@ -381,7 +381,7 @@ class GatedAttention(Attention):
             w_o = wide
         self.w_o = w_o.contiguous()
         if self.maps == 2:
-            # one number for the layer, formed once in float32
+            # a scalar of the layer, formed once in float32
             l1 = (f32(tensors[n["lq1"]]) * f32(tensors[n["lk1"]])).sum()
             l2 = (f32(tensors[n["lq2"]]) * f32(tensors[n["lk2"]])).sum()
             self.lam = float(torch.exp(l1) - torch.exp(l2)) + self.diff
