@@ -33,7 +33,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # bfloat16 engine can avoid) then moves a row by 1.7e-2 at worst, where the untamed model moves by 1.2e-1.
 TOL = {"float32": 1e-3, "bfloat16": 1e-1}
 LENGTHS = {"A": [70, 133, 33, 200, 97, 64], "B": [1, 9, 40, 100, 150, 57], "odd": [31, 2, 77, 50],
-           "loop_all": [30, 3, 66], "loop_one": [45, 8, 90, 2], "attention": [40, 75, 130, 9], "diff": [40, 75, 130, 9],
+           "loop_all": [30, 3, 66], "loop_one": [45, 8, 90, 2], "wide": [50, 7, 101], "attention": [40, 75, 130, 9], "diff": [40, 75, 130, 9],
            "delta": [24, 121, 48, 5], "moe": [24, 121, 48, 5]}
 
 _cache = {}
@@ -110,8 +110,8 @@ def all_free(runner):
         runner.cache.free_slots == runner.cache.max_seqs
 
 
-CASES = [(n, "float32") for n in ("attention", "diff", "delta", "moe", "loop_all", "loop_one", "A", "B", "odd")] + \
-        [(n, "bfloat16") for n in ("attention", "diff", "delta", "moe", "loop_one", "A", "B")]
+CASES = [(n, "float32") for n in ("attention", "diff", "delta", "moe", "loop_all", "loop_one", "wide", "A", "B", "odd")] + \
+        [(n, "bfloat16") for n in ("attention", "diff", "delta", "moe", "loop_one", "wide", "A", "B")]
 
 
 @pytest.mark.parametrize("name,dtype", CASES)

@@ -86,13 +86,17 @@ ODD = model(50, 199, [
     layer(attention_2(2, 2, 6, 11, 13, 4, 0.25, 777.0), moe(2, 1, 7)),
 ], loop=(0, 2, 2), scale=0.5)
 
+# heads beyond what the matrix-core attention kernels take: the general kernel in both precisions
+WIDE = model(64, 199, [layer(attention(2, 1, 136, 200, (0.3, 11)), moe(3, 2, 16)),
+                       layer(attention_2(2, 2, 40, 144, 33, 20, 0.4), None)], loop=(1, 2, 2))
+
 ONLY_ATTENTION = model(64, 199, [layer(attention(6, 2, 16, 8, (0.8, 8)), None)])
 ONLY_DIFF = model(64, 199, [layer(attention_2(4, 2, 16, 24, 20, 8), None)])
 ONLY_DELTA = model(64, 199, [layer(delta(4, 2, 16, 24, 4), None)])
 ONLY_MOE = model(64, 199, [layer(attention(2, 2, 8, 8, None), moe(8, 3, 16))])
 
 CONFIGS = {"A": (MIX_A, 16), "B": (MIX_B, 8), "loop_all": (LOOP_ALL, 4), "loop_one": (LOOP_ONE, 16), "odd": (ODD, 4),
-           "attention": (ONLY_ATTENTION, 4), "diff": (ONLY_DIFF, 8), "delta": (ONLY_DELTA, 16), "moe": (ONLY_MOE, 16)}
+           "wide": (WIDE, 16), "attention": (ONLY_ATTENTION, 4), "diff": (ONLY_DIFF, 8), "delta": (ONLY_DELTA, 16), "moe": (ONLY_MOE, 16)}
 
 
 def every_expert(cfg):

@@ -293,8 +293,8 @@ class GatedAttention(Attention):
         if dim <= 0 or vdim <= 0:
             raise ValueError(f"{prefix}: head_dim and value_dim must be positive")
         D = max(dim, vdim)
-        if -(-D // 16) * 16 <= 128:
-            D = -(-D // 16) * 16
+        # a multiple of 16 where the matrix-core kernels take the head (up to 128), else of 8 (rows of 16 bytes)
+        D = -(-D // 16) * 16 if -(-D // 16) * 16 <= 128 else -(-D // 8) * 8
         if window and chunk:
             raise ValueError(f"{prefix}: a window or a chunked mask, not both")
         if int(window) < 0 or int(chunk) < 0:
