@@ -131,15 +131,16 @@ __global__ void norm_prescale_kernel(const float* __restrict__ x, const TW* __re
 }
 
 // ------------------------------------------------------------------ SiLU-gate
-// z[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]
+// z[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]; with `pairs` the row holds (gate_j, up_j) side by side:
+// z[t, j] = silu(gate_up[t, 2j]) * gate_up[t, 2j + 1]
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ z, int64_t total, int inter) {
+__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ z, int64_t total, int inter, int pairs) {
   const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   if (i >= total) return;
   const int64_t t = i / inter;
   const int j = (int)(i - t * inter);
-  const float g = to_f32(gate_up[t * 2 * inter + j]);
-  const float u = to_f32(gate_up[t * 2 * inter + inter + j]);
+  const float g = to_f32(gate_up[t * 2 * inter + (pairs ? 2 * j : j)]);
+  const float u = to_f32(gate_up[t * 2 * inter + (pairs ? 2 * j + 1 : inter + j)]);
   z[i] = from_f32<T>(g / (1.f + expf(-g)) * u);
 }
 
@@ -379,12 +380,12 @@ int tl_norm_prescale(const float* x, const void* w, const int32_t* rows, void* o
   return tl_launch_status();
 }
 
-int tl_silu_mul(const void* gate_up, void* z, int n_tokens, int inter, int dtype, hipStream_t stream) {
+int tl_silu_mul(const void* gate_up, void* z, int n_tokens, int inter, int pairs, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
-  if (inter <= 0) return TL_ERR_ARG;
+  if (inter <= 0 || (pairs != 0 && pairs != 1)) return TL_ERR_ARG;
   const int64_t total = (int64_t)n_tokens * inter;
   TL_DISPATCH_T(dtype, hipLaunchKernelGGL(silu_mul_kernel<T>, dim3((unsigned)ceil_div64(total, kThreads)),
-                                          dim3(kThreads), 0, stream, (const T*)gate_up, (T*)z, total, inter);)
+                                          dim3(kThreads), 0, stream, (const T*)gate_up, (T*)z, total, inter, pairs);)
   return tl_launch_status();
 }
 

@@ -1979,18 +1979,22 @@ int tl_linear_handoff(const void* a, const void* w, void* out, const float* resi
 // out = a @ w[g]^T by runs of rows: a bfloat16 [M, K] whose aligned runs of `group_rows` rows (256: a multiple of
 // every tile height; M a multiple of it) each belong to one group g = tile_group[run] (negative: the run holds no
 // row and nothing is computed or written for it); w bfloat16 [groups, N, K]; out [M, N] bfloat16 or float32.
+// swiglu: the N columns are (gate_j, up_j) pairs and out [M, N / 2] (bfloat16) = silu(gate) * up.
 int tl_linear_grouped(const void* a, const void* w, void* out, const int32_t* tile_group, int group_rows, int M, int N,
-                      int K, int64_t lda, int64_t ldo, int out_dtype, hipStream_t stream) {
+                      int K, int64_t lda, int64_t ldo, int out_dtype, int swiglu, hipStream_t stream) {
   if (M <= 0) return TL_OK;
-  if (N <= 0 || K <= 0 || K % 8 || lda % 8 || lda < K || ldo < N || (out_dtype != 0 && out_dtype != 1) || !tile_group ||
-      group_rows != 256 || M % group_rows || !a || !w || !out)
+  if (N <= 0 || K <= 0 || K % 8 || lda % 8 || lda < K || ldo < (swiglu ? N / 2 : N) || (out_dtype != 0 && out_dtype != 1) ||
+      !tile_group || group_rows != 256 || M % group_rows || !a || !w || !out || (swiglu && (out_dtype != 1 || (N & 1))))
     return TL_ERR_ARG;
   TileNorm nm;
   nm.tile_group = tile_group;
   nm.group_rows = group_rows;
   nm.group_stride = (int64_t)N * K;
   int rc;
-  if (out_dtype == 0)
+  if (swiglu)
+    rc = launch_gemm_bf16_any<bf16_t, true>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, nullptr, nm, M, N, K, lda,
+                                            ldo, 0, 0, stream);
+  else if (out_dtype == 0)
     rc = launch_gemm_bf16_any<float, false>((const bf16_t*)a, (const bf16_t*)w, (float*)out, nullptr, nm, M, N, K, lda,
                                             ldo, 0, 0, stream);
   else

@@ -125,8 +125,8 @@ __device__ __forceinline__ float activate(float v, int act) {
 }
 
 // out[t * top + j, n] = act(sum_k a[t, k] * w[e(t, j)][n, k]); with the gated activation an expert's N rows are
-// [gate rows | up rows] and out[t * top + j, n] = silu(gate_n) * up_n for n < N / 2, formed from the float32 sums
-// (a wave's four dot products are then two gates and their two ups).
+// (gate_0, up_0, gate_1, up_1, ...) and out[t * top + j, n] = silu(gate_n) * up_n for n < N / 2, formed from the
+// float32 sums (a wave's four dot products are then two gates and their two ups).
 template <typename T>
 __global__ __launch_bounds__(kThreads) void table_moe_up_kernel(const T* __restrict__ a, int64_t a_stride,
                                                                 const T* __restrict__ w,
@@ -145,11 +145,11 @@ __global__ __launch_bounds__(kThreads) void table_moe_up_kernel(const T* __restr
     for (int n = n0; n < min(F, n0 + kCols / kWaves); n += 2) {
       const T* wr[4];
 #pragma unroll
-      for (int c = 0; c < 4; ++c) wr[c] = we + (int64_t)((c / 2) * F + min(n + (c & 1), F - 1)) * K;
+      for (int c = 0; c < 4; ++c) wr[c] = we + (int64_t)(2 * min(n + c / 2, F - 1) + (c & 1)) * K;
       float v[4];
       dot_lanes4(arow, wr, K, lane, v);
       if (lane < 2 && n + lane < F) {
-        const float g = v[lane], u = v[lane + 2];
+        const float g = v[2 * lane], u = v[2 * lane + 1];
         out[(int64_t)row * F + n + lane] = from_f32<T>(g / (1.f + expf(-g)) * u);
       }
     }

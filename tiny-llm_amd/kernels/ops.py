@@ -536,16 +536,17 @@ def linear_handoff(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual
     return out
 
 
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]."""
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, pairs: bool = False) -> torch.Tensor:
+    """out[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]; pairs: the rows hold (gate_j, up_j) side by side and
+    out[t, j] = silu(gate_up[t, 2j]) * gate_up[t, 2j + 1]."""
     _dev(gate_up, out)
     T, I2 = gate_up.shape
     if not (I2 % 2 == 0 and gate_up.is_contiguous()):
         _fail("gate_up must be contiguous [T, 2I]")
     if not (out.dtype == gate_up.dtype and out.is_contiguous() and tuple(out.shape) == (T, I2 // 2)):
         _fail("silu_mul output must be contiguous [T, I] of the input's type")
-    _check(_lib().tl_silu_mul(_ptr(gate_up), _ptr(out), c_int(T), c_int(I2 // 2), c_int(_dt(gate_up)),
-                              _stream()), "silu_mul")
+    _check(_lib().tl_silu_mul(_ptr(gate_up), _ptr(out), c_int(T), c_int(I2 // 2), c_int(1 if pairs else 0),
+                              c_int(_dt(gate_up)), _stream()), "silu_mul")
     return out
 
 
@@ -1840,15 +1841,15 @@ def tanh_rows(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 
 # ------------------------------------------------------------ experts looked up in a table
 MOE_ACTIVATIONS = {None: 0, "relu2": 1}      # what may follow an expert's first product (csrc/moe.hip)
-MOE_GATED = "swiglu"                         # `table_moe_up` only: an expert's rows are [gate | up], out = silu(gate) * up
+MOE_GATED = "swiglu"                         # `table_moe_up` only: an expert's rows are (gate_j, up_j) pairs, out = silu(gate) * up
 
 
 def table_moe_up(a: torch.Tensor, w: torch.Tensor, tokens: Optional[torch.Tensor], table: torch.Tensor, out: torch.Tensor,
                  act: Optional[str] = None) -> torch.Tensor:
     """out[t * top + j] = act(w[table[tokens[t], j]] @ a[t]); a [T, K], w [E, N, K] of one type, table int32 [vocab, top],
     out contiguous [T * top, N].  tokens None: the table has a row per row of a (the experts a router chose).
-    act None, "relu2" (the square of max(., 0)) or "swiglu": an expert's N rows are [gate rows | up rows] and out
-    [T * top, N / 2] = silu(gate) * up, formed from the float32 sums."""
+    act None, "relu2" (the square of max(., 0)) or "swiglu": an expert's N rows are (gate_0, up_0, gate_1, up_1, ...) and
+    out [T * top, N / 2] = silu(gate) * up, formed from the float32 sums."""
     _dev(a, w, tokens, table, out)
     _need(act in MOE_ACTIVATIONS or act == MOE_GATED, f"table_moe_up: activation {act!r} is not built")
     _rows_2d(a, "table_moe_up input")
@@ -1973,10 +1974,13 @@ def moe_gather(a: Optional[torch.Tensor], a_div: int, plan: torch.Tensor, rows: 
                                 _stream()), "moe_gather")
 
 
-def linear_grouped(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def linear_grouped(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, out: torch.Tensor,
+                   epilogue: Optional[str] = None) -> torch.Tensor:
     """out = a @ w[g]^T by runs of 256 rows: run r of a (bfloat16 [runs * 256, K]) multiplies w[tile_group[r]]
     (bfloat16 [G, N, K]); a run whose entry is negative is skipped (its rows of out are not written).  out
-    [runs * 256, N] bfloat16 or float32.  The tiled product of `linear` with a weight matrix per run of rows."""
+    [runs * 256, N] bfloat16 or float32.  The tiled product of `linear` with a weight matrix per run of rows.
+    epilogue="swiglu" as there: the N columns are (gate_j, up_j) pairs and out [runs * 256, N / 2] (bfloat16) =
+    silu(gate) * up, from the float32 accumulators."""
     _dev(a, w, tile_group, out)
     _rows_2d(a, "linear_grouped input")
     _rows_2d(out, "linear_grouped output")
@@ -1985,12 +1989,17 @@ def linear_grouped(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, o
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.is_contiguous() and w.shape[2] == K,
           "linear_grouped: a [M, K] and contiguous w [G, N, K] are bfloat16")
     _need(M % MOE_RUN_ROWS == 0 and K % 8 == 0 and a.stride(0) % 8 == 0, "linear_grouped: runs of 256 rows, K a multiple of 8")
-    _need(tuple(out.shape) == (M, N), "linear_grouped: out is [M, N]")
+    swiglu = _epilogue(epilogue)
+    if swiglu:
+        _need(N % 2 == 0 and tuple(out.shape) == (M, N // 2) and out.dtype == torch.bfloat16,
+              "linear_grouped: the SiLU-gate epilogue writes bfloat16 [M, N / 2]")
+    else:
+        _need(tuple(out.shape) == (M, N), "linear_grouped: out is [M, N]")
     _i32(tile_group)
     _need(tile_group.numel() >= M // MOE_RUN_ROWS, "linear_grouped: one group per run of rows")
     _check(_lib().tl_linear_grouped(_ptr(a, 16), _ptr(w, 16), _ptr(out, 16), _ptr(tile_group), c_int(MOE_RUN_ROWS),
                                     c_int(M), c_int(N), c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)),
-                                    c_int(_dt(out)), _stream()), "linear_grouped")
+                                    c_int(_dt(out)), c_int(swiglu), _stream()), "linear_grouped")
     return out
 
 

@@ -186,9 +186,10 @@ class RoutedMoE(FeedForward):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         p, E = self.prefix, self.num_experts
-        if self.gated:      # an expert's first product gives [gate | up]
-            self.w_up = torch.stack([torch.cat([tensors[f"{p}.e{e}.gate"], tensors[f"{p}.e{e}.up"]], dim=0)
-                                     for e in range(E)]).contiguous()
+        if self.gated:      # an expert's first product gives (gate_0, up_0, gate_1, up_1, ...): rows interleaved, as in
+            # the dense gated layer, so that a product's epilogue sees each pair in one lane
+            self.w_up = torch.stack([torch.stack([tensors[f"{p}.e{e}.gate"], tensors[f"{p}.e{e}.up"]], dim=1)
+                                     .reshape(2 * self.intermediate_size, self.hidden_size) for e in range(E)]).contiguous()
         else:
             self.w_up = torch.stack([tensors[f"{p}.e{e}.up"] for e in range(E)]).contiguous()
         self.w_down = torch.stack([tensors[f"{p}.e{e}.down"] for e in range(E)]).contiguous()
@@ -243,10 +244,8 @@ class RoutedMoE(FeedForward):
             pos = ops.scratch("moe_row_pos", (rows,), torch.int32, dev)
             ops.moe_gather(h, top, plan, rows, E, R, hp, pos)
             z = ops.scratch("moe_gated", (cap, F), self.dtype, dev)
-            if self.gated:
-                gup = ops.scratch("moe_gate_up", (cap, 2 * F), self.dtype, dev)
-                ops.linear_grouped(hp, self.w_up, runs, gup)
-                ops.silu_mul(gup, z)
+            if self.gated:      # the gate in the product's epilogue
+                ops.linear_grouped(hp, self.w_up, runs, z, epilogue="swiglu")
             else:
                 up = ops.scratch("moe_up", (cap, F), torch.float32, dev)        # float32: rounded once, behind the activation
                 ops.linear_grouped(hp, self.w_up, runs, up)
@@ -262,7 +261,7 @@ class RoutedMoE(FeedForward):
             if self.gated:
                 gup = ops.scratch("moe_gate_up", (rows, 2 * F), self.dtype, dev)
                 ops.grouped_rows_gemm(h, top, self.w_up, plan, gup)
-                ops.silu_mul(gup, z)
+                ops.silu_mul(gup, z, pairs=True)
             else:
                 up = ops.scratch("moe_up", (rows, F), torch.float32, dev)
                 ops.grouped_rows_gemm(h, top, self.w_up, plan, up)
