@@ -357,12 +357,13 @@ ATTENTION_KERNELS = ["general float32", "general bfloat16", "matrix cores float3
 
 
 @pytest.mark.parametrize("kernel", ATTENTION_KERNELS)
-@pytest.mark.parametrize("chunk", [40, 1, 17, 64, 150])
+@pytest.mark.parametrize("chunk", [40, 1, 17, 64, 150, 0])
 def test_chunked_mask_finds_one_key(kernel, chunk):
     """One query per place of interest is aligned with one key (and scaled so that this score stands out): the result
     must be that key's value.  Keys at the chunk's first place, at both sides of page edges, the query's own position,
     the first positions; the key just OUTSIDE the chunk (the last of the chunk before) and the one behind the query
-    are louder still, and the mask must hide them.  Every attention kernel takes the chunk as a negative window."""
+    are louder still, and the mask must hide them.  Every attention kernel takes the chunk as a negative window.
+    Chunk 0 is no chunk at all (the mixer without a mask): the one key then lies hundreds of positions back."""
     from tiny_llm_amd.kernels import ops
     dtype = torch.float32 if "float32" in kernel else torch.bfloat16
     g = torch.Generator().manual_seed(5)
@@ -372,9 +373,9 @@ def test_chunked_mask_finds_one_key(kernel, chunk):
     vals = torch.randn(n, kvh, d, generator=g)
     table = torch.randperm(64, generator=g)[: -(-n // block)].tolist()
     k_pages, v_pages = _paged_kv(keys, table, block, 64, dtype), _paged_kv(vals, table, block, 64, dtype)
-    first = lambda pos: pos // chunk * chunk
+    first = lambda pos: pos // chunk * chunk if chunk else 0
     places = {699, 650, 640, 639, 600, 599, 400, 399, 200, 199, 64, 63, 48, 47, 31, 16, 15, 1, 0,
-              first(699), first(699) - 1, first(300), first(300) + chunk - 1}
+              first(699), first(699) - 1, first(300), first(300) + chunk - 1, 300}
     cases = sorted({(pos, key) for pos in places if 0 <= pos < n
                     for key in (first(pos), pos, (first(pos) + pos) // 2, min(first(pos) + 1, pos))})
     T = len(cases)
